@@ -1,0 +1,90 @@
+/*
+ * C ABI of the MI355X (gfx950) packed-int4 GEMM library, libqm_hip.so.
+ *
+ *   C[M,N] (int32, row-major) = A[M,K] (s4) * B[N,K]^T (s4)
+ *
+ * A and B are packed two nibbles per byte along K: byte j of a row holds element
+ * 2j in bits 0..3 and element 2j+1 in bits 4..7, two's complement (reference:
+ * pack_b, test.py:6-15; unpack_int4_matrix, kernel.cu:389-408).  A is [M, K/2]
+ * bytes, B is [N, K/2] bytes ("B is transposed", kernel.cu:78), C is fully
+ * overwritten (kernel.cu:99-114,173).
+ *
+ * Plain pointers and sizes only; every pointer is a DEVICE pointer borrowed for
+ * the duration of the enqueued work; `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream).  Every call is asynchronous, allocates nothing,
+ * never synchronises and is therefore safe under HIP graph capture, as the
+ * reference's harness requires (test.py:78-81).
+ *
+ * Every function returning int returns QM_OK (0) or a negative QM_ERR_* code;
+ * qm_status_string() names it.  The reference has no error reporting at all
+ * (extension.cpp:11-15 commented out, kernel.cu:282-288 commented out, unknown
+ * shapes silently skipped at kernel.cu:340-385); returning a status is a
+ * deliberate strengthening.
+ */
+#ifndef QM_ABI_H
+#define QM_ABI_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QM_OK                 0
+#define QM_ERR_NULL          -1 /* a required pointer is NULL                               */
+#define QM_ERR_SHAPE         -2 /* m, n or k negative, k odd, or a size overflows int32     */
+#define QM_ERR_CONFIG        -3 /* cfg id unknown, or that config cannot run this shape     */
+#define QM_ERR_LAUNCH        -4 /* the HIP runtime refused the launch (see qm_last_hip_error) */
+#define QM_ERR_ALIGN         -5 /* C is not 4-byte aligned                                  */
+
+#define QM_CFG_AUTO          -1 /* let the shape table / heuristic choose                   */
+
+/*
+ * The hot path.  Replaces
+ *   void wrapper(void *A, void *B, void *C, const int m, const int n, const int k,
+ *                cudaStream_t stream)                 (kernel.cu:334, declared extension.cpp:6)
+ * with the same seven arguments in the same order plus a status.  Unlike the
+ * reference, every shape with m,n >= 0 and even k >= 0 is computed (m or n == 0
+ * is a no-op, k == 0 zero-fills C).
+ */
+int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, int k, void *stream);
+
+/*
+ * Same, with an explicit kernel configuration.  Replaces the compile-time choice
+ * made by LAUNCH_KERNEL_IF_CONDITION / IGemmConfig (kernel.cu:321-332, 23-50)
+ * from the constexpr table in configs.cu:19-689; used by the autotuner that
+ * regenerates this library's per-shape table.  cfg = QM_CFG_AUTO behaves as
+ * qm_gemm_i4.
+ */
+int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg);
+
+/* The configuration qm_gemm_i4 would pick for this shape (the table lookup the
+ * reference does at kernel.cu:340-385, here with a heuristic fallback instead of
+ * a silent no-op).  ptr_align is the smallest alignment in bytes shared by A and
+ * B (pass 16 or more when they come from a device allocator). */
+int qm_select_config(int m, int n, int k, int ptr_align);
+
+/* Introspection of the compiled-in configurations (the counterpart of the
+ * KernelConfig instances, configs.cu:1-17). */
+int         qm_num_configs(void);
+const char *qm_config_name(int cfg);                       /* NULL when cfg is out of range */
+int         qm_config_supports(int cfg, int m, int n, int k, int ptr_align); /* 1 / 0      */
+
+/*
+ * Device-side packing and unpacking, the steps on either side of the GEMM:
+ *   qm_pack_i4   replaces pack_b (test.py:6-15):             [rows,K] int8 -> [rows,K/2] bytes
+ *   qm_unpack_i4 replaces unpack_int4_matrix (kernel.cu:389-408): the inverse
+ * Values outside [-8,7] are truncated to their low nibble when packing.
+ */
+int qm_pack_i4(const void *src_i8, void *dst_packed, int rows, int k, void *stream);
+int qm_unpack_i4(const void *src_packed, void *dst_i8, int rows, int k, void *stream);
+
+/* Diagnostics. */
+const char *qm_status_string(int status);
+int         qm_last_hip_error(void);      /* hipError_t of the last failed launch on this thread */
+const char *qm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QM_ABI_H */

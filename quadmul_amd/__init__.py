@@ -1,0 +1,220 @@
+"""quadmul_amd: packed-int4 GEMM for MI355X (gfx950), host-side interface.
+
+Two ways in, both ending in the same C ABI (``include/qm_abi.h``,
+``quadmul_amd/lib/libqm_hip.so``):
+
+* the PyTorch-ROCm extension module ``quadmul`` (repo root), the drop-in for the
+  reference's module of the same name: ``quadmul.gemm(a, b, c, m, n, k)``
+  (extension.cpp:8-29, call site test.py:40);
+* this package, which binds the C ABI with ctypes and takes torch tensors only to
+  borrow their device pointers and the current stream.
+
+There is no CPU or eager fallback for the GEMM: if the HIP library has not been
+built, every call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import List, Optional
+
+import torch
+
+__all__ = [
+    "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "pack_int4", "unpack_int4",
+    "num_configs", "config_name", "config_names", "config_id", "select_config", "config_supports",
+    "CFG_AUTO", "version",
+]
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_PKG, "lib", "libqm_hip.so")
+_lib: Optional[ctypes.CDLL] = None
+
+CFG_AUTO = -1
+#: every symbol include/qm_abi.h declares
+ABI_SYMBOLS = (
+    "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_select_config", "qm_num_configs", "qm_config_name",
+    "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version",
+)
+
+
+class QuadmulError(RuntimeError):
+    """A non-zero status from libqm_hip.so."""
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def library() -> ctypes.CDLL:
+    """The loaded C-ABI library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise QuadmulError(
+            f"{_LIB_PATH} is missing: build it with `python -m quadmul_amd.build` "
+            "(there is no fallback path for the int4 GEMM)")
+    lib = ctypes.CDLL(_LIB_PATH)
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.qm_gemm_i4.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+    lib.qm_gemm_i4.restype = ci
+    lib.qm_gemm_i4_cfg.argtypes = [vp, vp, vp, ci, ci, ci, vp, ci]
+    lib.qm_gemm_i4_cfg.restype = ci
+    lib.qm_select_config.argtypes = [ci, ci, ci, ci]
+    lib.qm_select_config.restype = ci
+    lib.qm_num_configs.argtypes = []
+    lib.qm_num_configs.restype = ci
+    lib.qm_config_name.argtypes = [ci]
+    lib.qm_config_name.restype = ctypes.c_char_p
+    lib.qm_config_supports.argtypes = [ci, ci, ci, ci, ci]
+    lib.qm_config_supports.restype = ci
+    lib.qm_pack_i4.argtypes = [vp, vp, ci, ci, vp]
+    lib.qm_pack_i4.restype = ci
+    lib.qm_unpack_i4.argtypes = [vp, vp, ci, ci, vp]
+    lib.qm_unpack_i4.restype = ci
+    lib.qm_status_string.argtypes = [ci]
+    lib.qm_status_string.restype = ctypes.c_char_p
+    lib.qm_last_hip_error.argtypes = []
+    lib.qm_last_hip_error.restype = ci
+    lib.qm_version.argtypes = []
+    lib.qm_version.restype = ctypes.c_char_p
+    _lib = lib
+    return lib
+
+
+def _check(status: int, what: str) -> None:
+    if status == 0:
+        return
+    lib = library()
+    msg = lib.qm_status_string(status).decode()
+    if status == -4:
+        msg += f" (hipError_t {lib.qm_last_hip_error()})"
+    raise QuadmulError(f"{what}: {msg}")
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _is_byte(t: torch.Tensor) -> bool:
+    return t.dtype in (torch.int8, torch.uint8)
+
+
+def _check_operands(a, b, c, m, n, k) -> None:
+    # The checks the reference left commented out (extension.cpp:11-15).
+    if not (a.is_cuda and b.is_cuda and c.is_cuda):
+        raise QuadmulError("gemm: a, b and c must be GPU tensors")
+    if not (a.device == b.device == c.device):
+        raise QuadmulError("gemm: all tensors must be on the same device")
+    if not (_is_byte(a) and _is_byte(b)):
+        raise QuadmulError("gemm: a and b must be int8 or uint8 (packed int4)")
+    if c.dtype != torch.int32:
+        raise QuadmulError("gemm: c must be int32")
+    if not (a.is_contiguous() and b.is_contiguous() and c.is_contiguous()):
+        raise QuadmulError("gemm: all tensors must be contiguous")
+    if m < 0 or n < 0 or k < 0 or k % 2:
+        raise QuadmulError("gemm: m, n, k must be >= 0 and k even")
+    if a.numel() != m * (k // 2) or b.numel() != n * (k // 2) or c.numel() != m * n:
+        raise QuadmulError("gemm: tensor sizes do not match m, n, k")
+
+
+def gemm_cfg(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int, cfg: int = CFG_AUTO) -> None:
+    """``c[m,n] = a[m,k] @ b[n,k].T`` on packed int4, with an explicit kernel configuration.
+
+    ``cfg``: config id in the low 16 bits, tile-raster group height in bits 16..23
+    (0 = default); ``CFG_AUTO`` = table / cost model.
+    """
+    _check_operands(a, b, c, m, n, k)
+    with torch.cuda.device(a.device):
+        st = library().qm_gemm_i4_cfg(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, _stream_ptr(a), cfg)
+    _check(st, "qm_gemm_i4_cfg")
+
+
+def gemm(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int) -> None:
+    """Same contract as the reference's ``quadmul.gemm`` (extension.cpp:8-24): ``a`` is
+    packed A ``[m, k/2]``, ``b`` is packed B stored ``[n, k/2]``, ``c`` is ``[m, n]`` int32
+    and is overwritten; enqueued on the current stream of ``a``'s device; returns None."""
+    _check_operands(a, b, c, m, n, k)
+    with torch.cuda.device(a.device):
+        st = library().qm_gemm_i4(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, _stream_ptr(a))
+    _check(st, "qm_gemm_i4")
+
+
+def pack_int4(values: torch.Tensor) -> torch.Tensor:
+    """``[rows, K]`` int8 holding int4 values -> ``[rows, K/2]`` int8, even k in the low
+    nibble: the reference's ``pack_b`` (test.py:6-15).  GPU tensors are packed by the
+    library's kernel, CPU tensors with the same bit arithmetic in torch."""
+    if values.dtype != torch.int8 or values.dim() != 2:
+        raise QuadmulError("pack_int4: expects a 2-D int8 tensor")
+    rows, k = values.shape
+    if k % 2:
+        raise QuadmulError("pack_int4: K must be even")
+    v = values.contiguous()
+    if v.is_cuda:
+        out = torch.empty((rows, k // 2), dtype=torch.int8, device=v.device)
+        with torch.cuda.device(v.device):
+            st = library().qm_pack_i4(v.data_ptr(), out.data_ptr(), rows, k, _stream_ptr(v))
+        _check(st, "qm_pack_i4")
+        return out
+    u = v.view(torch.uint8).reshape(-1)
+    return ((u[0::2] & 0x0F) | ((u[1::2] & 0x0F) << 4)).reshape(rows, k // 2).view(torch.int8).contiguous()
+
+
+def unpack_int4(packed: torch.Tensor) -> torch.Tensor:
+    """``[rows, K/2]`` bytes -> ``[rows, K]`` int8: the reference's ``unpack_int4_matrix``
+    (kernel.cu:389-408)."""
+    if not _is_byte(packed) or packed.dim() != 2:
+        raise QuadmulError("unpack_int4: expects a 2-D int8/uint8 tensor")
+    p = packed.contiguous()
+    rows, half = p.shape
+    if p.is_cuda:
+        out = torch.empty((rows, 2 * half), dtype=torch.int8, device=p.device)
+        with torch.cuda.device(p.device):
+            st = library().qm_unpack_i4(p.data_ptr(), out.data_ptr(), rows, 2 * half, _stream_ptr(p))
+        _check(st, "qm_unpack_i4")
+        return out
+    u = p.view(torch.uint8)
+    lo = (u & 0x0F).to(torch.int16)
+    hi = (u >> 4).to(torch.int16)
+    lo = torch.where(lo > 7, lo - 16, lo)
+    hi = torch.where(hi > 7, hi - 16, hi)
+    return torch.stack((lo, hi), dim=2).reshape(rows, 2 * half).to(torch.int8)
+
+
+def num_configs() -> int:
+    return int(library().qm_num_configs())
+
+
+def config_name(cfg: int) -> str:
+    s = library().qm_config_name(cfg)
+    if s is None:
+        raise QuadmulError(f"no kernel configuration {cfg}")
+    return s.decode()
+
+
+def config_names() -> List[str]:
+    return [config_name(i) for i in range(num_configs())]
+
+
+def config_id(name: str) -> int:
+    names = config_names()
+    if name not in names:
+        raise QuadmulError(f"no kernel configuration named {name!r}")
+    return names.index(name)
+
+
+def select_config(m: int, n: int, k: int, ptr_align: int = 256) -> int:
+    """The (config id | group_m << 16) ``gemm`` would use for this shape."""
+    v = int(library().qm_select_config(m, n, k, ptr_align))
+    if v < 0:
+        _check(v, "qm_select_config")
+    return v
+
+
+def config_supports(cfg: int, m: int, n: int, k: int, ptr_align: int = 256) -> bool:
+    return bool(library().qm_config_supports(cfg, m, n, k, ptr_align))
+
+
+def version() -> str:
+    return library().qm_version().decode()

@@ -1,0 +1,115 @@
+"""Build recipe for the gfx950 library and the PyTorch-ROCm extension, in-tree.
+
+    python -m quadmul_amd.build            # both
+    python -m quadmul_amd.build --lib      # libqm_hip.so only (hipcc, no torch needed)
+
+Outputs (git-ignored, but they travel with the tree):
+    quadmul_amd/lib/libqm_hip.so                      hand-written HIP kernels + C ABI
+    quadmul.cpython-<abi>.so  (repo root)             module `quadmul`, host-only C++
+
+The kernels are compiled by hipcc for gfx950 only; the extension is compiled by
+the host compiler against torch's headers and calls the library through
+include/qm_abi.h.  Takes the place of the reference's setup.py:1-17 (nvcc +
+CUDAExtension), without torch's source-translation step.
+"""
+from __future__ import annotations
+
+import argparse
+import os
+import shutil
+import subprocess
+import sys
+import sysconfig
+from concurrent.futures import ThreadPoolExecutor
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIBDIR = os.path.join(PKG, "lib")
+OBJDIR = os.path.join(PKG, "build")
+LIB_PATH = os.path.join(LIBDIR, "libqm_hip.so")
+N_TILE_TUS = 8
+
+HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+]
+
+
+def ext_path() -> str:
+    return os.path.join(ROOT, "quadmul" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + out)
+    return out
+
+
+def build_lib(jobs: int = 8, verbose: bool = False) -> str:
+    os.makedirs(LIBDIR, exist_ok=True)
+    os.makedirs(OBJDIR, exist_ok=True)
+    units = [("qm_dispatch.o", ["-c", os.path.join(CSRC, "qm_dispatch.hip")])]
+    for tu in range(N_TILE_TUS):
+        units.append((f"qm_tile_inst_{tu}.o", [f"-DQM_TU={tu}", "-c", os.path.join(CSRC, "qm_tile_inst.hip")]))
+    objs = [os.path.join(OBJDIR, name) for name, _ in units]
+
+    def compile_one(item):
+        (name, args), obj = item
+        return _run([HIPCC] + HIP_FLAGS + args + ["-o", obj])
+
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, 16))) as pool:
+        for out in pool.map(compile_one, zip(units, objs)):
+            if verbose and out.strip():
+                print(out)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs)
+    return LIB_PATH
+
+
+def build_ext(verbose: bool = False) -> str:
+    import torch
+    from torch.utils import cpp_extension
+
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("build libqm_hip.so first")
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    incs = cpp_extension.include_paths() + [os.path.join(rocm, "include"), os.path.join(ROOT, "include"), sysconfig.get_paths()["include"]]
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=quadmul", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-Wno-deprecated-declarations"]
+    for i in incs:
+        cmd += ["-isystem", i]
+    cmd += [os.path.join(CSRC, "ext.cpp"), "-o", ext_path(),
+            "-L", LIBDIR, "-lqm_hip", "-L", torch_lib, "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip",
+            "-Wl,-rpath,$ORIGIN/quadmul_amd/lib", "-Wl,-rpath," + torch_lib]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return ext_path()
+
+
+def build_all(jobs: int = 8, verbose: bool = False):
+    return build_lib(jobs, verbose), build_ext(verbose)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--lib", action="store_true", help="build only libqm_hip.so")
+    ap.add_argument("--ext", action="store_true", help="build only the torch extension")
+    ap.add_argument("-j", "--jobs", type=int, default=8)
+    ap.add_argument("-v", "--verbose", action="store_true")
+    a = ap.parse_args(argv)
+    if a.lib or not a.ext:
+        print("built", build_lib(a.jobs, a.verbose))
+    if a.ext or not a.lib:
+        print("built", build_ext(a.verbose))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,95 @@
+// PyTorch-ROCm extension module `quadmul`: the drop-in for the reference's
+// pybind11 module (extension.cpp:8-29) -- same module name (setup.py:8,11), same
+// function gemm(a, b, c, m, n, k) -> None, same positional order (test.py:40).
+// Host-only C++: tensors are unwrapped to device pointers and handed, with the
+// current HIP stream of a's device (extension.cpp:23), to the C ABI in
+// include/qm_abi.h.  No kernels and no HIP runtime calls live here.
+//
+// The argument checks the reference left commented out (extension.cpp:11-15) are
+// live here; a non-zero status from the library is raised as RuntimeError.
+#include <torch/extension.h>
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include "qm_abi.h"
+
+namespace {
+
+void check_status(int status, const char *what)
+{
+    if (status == QM_OK) return;
+    if (status == QM_ERR_LAUNCH)
+        TORCH_CHECK(false, what, ": ", qm_status_string(status), " (hipError_t ", qm_last_hip_error(), ")");
+    TORCH_CHECK(false, what, ": ", qm_status_string(status));
+}
+
+bool is_byte(const torch::Tensor &t) { return t.scalar_type() == torch::kInt8 || t.scalar_type() == torch::kUInt8; }
+
+void *stream_of(const torch::Tensor &t) { return static_cast<void *>(c10::hip::getCurrentHIPStream(t.get_device()).stream()); }
+
+void check_operands(const torch::Tensor &a, const torch::Tensor &b, const torch::Tensor &c, int64_t m, int64_t n, int64_t k)
+{
+    TORCH_CHECK(a.is_cuda() && b.is_cuda() && c.is_cuda(), "quadmul.gemm: a, b and c must be GPU tensors");
+    TORCH_CHECK(a.device() == b.device() && a.device() == c.device(), "quadmul.gemm: all tensors must be on the same device");
+    // pack_b yields int8 (test.py:14); the reference only ever looks at data_ptr().
+    TORCH_CHECK(is_byte(a) && is_byte(b), "quadmul.gemm: a and b must be int8 or uint8 (packed int4)");
+    TORCH_CHECK(c.scalar_type() == torch::kInt32, "quadmul.gemm: c must be int32");
+    TORCH_CHECK(a.is_contiguous() && b.is_contiguous() && c.is_contiguous(), "quadmul.gemm: all tensors must be contiguous");
+    TORCH_CHECK(m >= 0 && n >= 0 && k >= 0 && k % 2 == 0, "quadmul.gemm: m, n, k must be >= 0 and k even");
+    TORCH_CHECK(m <= INT32_MAX && n <= INT32_MAX && k <= INT32_MAX, "quadmul.gemm: m, n, k must fit in int32");
+    TORCH_CHECK(a.numel() == m * (k / 2), "quadmul.gemm: a must hold m*k/2 bytes, got ", a.numel());
+    TORCH_CHECK(b.numel() == n * (k / 2), "quadmul.gemm: b must hold n*k/2 bytes, got ", b.numel());
+    TORCH_CHECK(c.numel() == m * n, "quadmul.gemm: c must hold m*n int32, got ", c.numel());
+}
+
+void gemm(torch::Tensor a, torch::Tensor b, torch::Tensor c, int64_t m, int64_t n, int64_t k)
+{
+    check_operands(a, b, c, m, n, k);
+    c10::OptionalDeviceGuard guard(a.device());
+    check_status(qm_gemm_i4(a.data_ptr(), b.data_ptr(), c.data_ptr(), (int)m, (int)n, (int)k, stream_of(a)), "quadmul.gemm");
+}
+
+void gemm_cfg(torch::Tensor a, torch::Tensor b, torch::Tensor c, int64_t m, int64_t n, int64_t k, int64_t cfg)
+{
+    check_operands(a, b, c, m, n, k);
+    c10::OptionalDeviceGuard guard(a.device());
+    check_status(qm_gemm_i4_cfg(a.data_ptr(), b.data_ptr(), c.data_ptr(), (int)m, (int)n, (int)k, stream_of(a), (int)cfg), "quadmul.gemm_cfg");
+}
+
+// Device-side pack_b (test.py:6-15): [rows, K] int8 -> [rows, K/2] int8.
+torch::Tensor pack(torch::Tensor values)
+{
+    TORCH_CHECK(values.is_cuda() && values.scalar_type() == torch::kInt8 && values.dim() == 2, "quadmul.pack: expects a 2-D int8 GPU tensor");
+    TORCH_CHECK(values.size(1) % 2 == 0, "quadmul.pack: K must be even");
+    auto v = values.contiguous();
+    c10::OptionalDeviceGuard guard(v.device());
+    auto out = torch::empty({v.size(0), v.size(1) / 2}, v.options());
+    check_status(qm_pack_i4(v.data_ptr(), out.data_ptr(), (int)v.size(0), (int)v.size(1), stream_of(v)), "quadmul.pack");
+    return out;
+}
+
+// Device-side unpack_int4_matrix (kernel.cu:389-408): [rows, K/2] bytes -> [rows, K] int8.
+torch::Tensor unpack(torch::Tensor packed)
+{
+    TORCH_CHECK(packed.is_cuda() && is_byte(packed) && packed.dim() == 2, "quadmul.unpack: expects a 2-D int8/uint8 GPU tensor");
+    auto p = packed.contiguous();
+    c10::OptionalDeviceGuard guard(p.device());
+    auto out = torch::empty({p.size(0), p.size(1) * 2}, p.options().dtype(torch::kInt8));
+    check_status(qm_unpack_i4(p.data_ptr(), out.data_ptr(), (int)p.size(0), (int)p.size(1) * 2, stream_of(p)), "quadmul.unpack");
+    return out;
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("gemm", &gemm, "Int4xInt4 Matrix Multiplication Kernel", py::arg("a"), py::arg("b"), py::arg("c"), py::arg("m"), py::arg("n"), py::arg("k"));
+    m.def("gemm_cfg", &gemm_cfg, "gemm with an explicit kernel configuration id (autotuning)");
+    m.def("pack", &pack, "Pack a [rows, K] int8 tensor of int4 values into [rows, K/2] bytes on the GPU");
+    m.def("unpack", &unpack, "Unpack [rows, K/2] bytes into a [rows, K] int8 tensor on the GPU");
+    m.def("num_configs", &qm_num_configs);
+    m.def("config_name", [](int cfg) { const char *s = qm_config_name(cfg); return std::string(s ? s : ""); });
+    m.def("select_config", &qm_select_config);
+    m.def("version", []() { return std::string(qm_version()); });
+}

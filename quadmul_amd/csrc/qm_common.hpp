@@ -1,0 +1,60 @@
+// Shared device helpers for the gfx950 packed-int4 GEMM kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace qm {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+struct GemmArgs {
+    const uint8_t *A;  // [M, K/2] packed s4
+    const uint8_t *B;  // [N, K/2] packed s4
+    int32_t *C;        // [M, N]
+    int M, N, K;
+};
+
+// gfx950 has no int4 MFMA, so nibbles are widened to int8 -- but scaled by 16,
+// which needs no per-byte sign fix-up.  For a dword w holding nibbles k0..k7
+// (k0 in bits 0..3), read as four int8 lanes:
+//     (w << 4) & 0xF0F0F0F0  ==  16 * s4(k0), 16 * s4(k2), 16 * s4(k4), 16 * s4(k6)
+//      w       & 0xF0F0F0F0  ==  16 * s4(k1), 16 * s4(k3), 16 * s4(k5), 16 * s4(k7)
+// because a nibble n placed in the high half of a byte is the int8 value 16*s4(n).
+// Both operands get the same treatment, so every int8 product carries a factor
+// 256 and the int32 accumulator holds exactly 256 * C; the epilogue shifts it out.
+// |C| <= 64 K, hence exact while 256 * 64 * K < 2^31, i.e. K <= QM_MAX_K_X16.
+// The even/odd split permutes K inside a dword; the contraction runs over K and
+// A and B are permuted identically, so the sum is unchanged.
+constexpr int QM_MAX_K_X16 = 131071;
+
+__device__ __forceinline__ int x16_even(int w) { return (int)(((uint32_t)w << 4) & 0xF0F0F0F0u); }
+__device__ __forceinline__ int x16_odd(int w) { return (int)((uint32_t)w & 0xF0F0F0F0u); }
+
+__device__ __forceinline__ void x16_expand(const v4i q, v4i &even, v4i &odd)
+{
+    even.x = x16_even(q.x); even.y = x16_even(q.y); even.z = x16_even(q.z); even.w = x16_even(q.w);
+    odd.x = x16_odd(q.x);   odd.y = x16_odd(q.y);   odd.z = x16_odd(q.z);   odd.w = x16_odd(q.w);
+}
+
+// D(16x16) += S0(16x64) * S1(64x16), int8 in, int32 out.  Lane l supplies row
+// l%16 of S0 / column l%16 of S1 for the 16 k-values of group l/16, and owns
+// D[4*(l/16) + r][l%16] in register r.
+__device__ __forceinline__ v4i mfma16(const v4i s0, const v4i s1, const v4i acc)
+{
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(s0, s1, acc, 0, 0, 0);
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs (id % 8), each with a private
+// L2.  Renumber so that every XCD owns one contiguous range of tile ids.
+__device__ __forceinline__ int xcd_contiguous_id(int bid, int nblocks)
+{
+    constexpr int XCDS = 8;
+    const int xcd = bid % XCDS, local = bid / XCDS;
+    const int per = (nblocks + XCDS - 1) / XCDS;  // size of the larger shares
+    const int tall = nblocks % XCDS;              // how many XCDs get a larger share (0: all equal)
+    if (tall == 0 || xcd < tall) return xcd * per + local;
+    return tall * per + (xcd - tall) * (per - 1) + local;
+}
+
+}  // namespace qm

@@ -1,0 +1,386 @@
+// C ABI of libqm_hip.so (include/qm_abi.h): argument checks, configuration
+// choice and launches.  Takes the place of the reference's host side:
+// wrapper (kernel.cu:334-385), LAUNCH_KERNEL_IF_CONDITION (kernel.cu:321-332)
+// and launch_igemm (kernel.cu:268-289).
+#include <atomic>
+#include <cstring>
+#include <mutex>
+
+#include "../../include/qm_abi.h"
+#include "qm_launch.hpp"
+#include "qm_skinny.hpp"
+
+#define QM_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace qm {
+
+// --------------------------------------------------------------------------
+// Fallback kernel: any M, N, even K, any alignment, no limit on K.  One thread
+// per element of C over LDS-staged 16x16x(128 nibble) tiles, plain byte loads.
+// --------------------------------------------------------------------------
+__device__ __forceinline__ int s4_lo(uint32_t b) { return (int)(int8_t)(b << 4) >> 4; }
+__device__ __forceinline__ int s4_hi(uint32_t b) { return (int)(int8_t)b >> 4; }
+
+__global__ void __launch_bounds__(256) gemm_generic_kernel(const GemmArgs p, const int tiles_n)
+{
+    __shared__ uint8_t As[16][64 + 4];
+    __shared__ uint8_t Bs[16][64 + 4];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int m0 = (blockIdx.x / tiles_n) * 16, n0 = (blockIdx.x % tiles_n) * 16;
+    const size_t Kb = (size_t)(p.K >> 1);
+    int32_t sum = 0;
+    for (size_t k0 = 0; k0 < Kb; k0 += 64) {
+        // 16 rows x 64 bytes per operand = 1024 bytes each, 4 bytes per thread
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int idx = threadIdx.x + t * 256, row = idx >> 6, col = idx & 63;
+            const bool kin = k0 + col < Kb;
+            As[row][col] = (kin && m0 + row < p.M) ? p.A[(size_t)(m0 + row) * Kb + k0 + col] : (uint8_t)0;
+            Bs[row][col] = (kin && n0 + row < p.N) ? p.B[(size_t)(n0 + row) * Kb + k0 + col] : (uint8_t)0;
+        }
+        __syncthreads();
+#pragma unroll 16
+        for (int j = 0; j < 64; ++j) {
+            const uint32_t a = As[ty][j], b = Bs[tx][j];
+            sum += s4_lo(a) * s4_lo(b) + s4_hi(a) * s4_hi(b);
+        }
+        __syncthreads();
+    }
+    if (m0 + ty < p.M && n0 + tx < p.N) p.C[(size_t)(m0 + ty) * p.N + n0 + tx] = sum;
+}
+
+static hipError_t launch_generic(const GemmArgs &p, hipStream_t stream, int)
+{
+    const long long tiles_m = (p.M + 15) / 16, tiles_n = (p.N + 15) / 16;
+    if (tiles_m * tiles_n > 0x7fffffffLL) return hipErrorInvalidValue;
+    gemm_generic_kernel<<<dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, stream>>>(p, (int)tiles_n);
+    return hipGetLastError();
+}
+
+// --------------------------------------------------------------------------
+// Zero fill (k == 0) and pack / unpack, flat over the whole array: K is even so
+// a byte never straddles two rows.
+// --------------------------------------------------------------------------
+__global__ void fill_zero_kernel(int32_t *dst, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = 0;
+}
+
+// 16 int8 in -> 8 packed bytes out per thread when aligned, else one byte per thread.
+__device__ __forceinline__ uint32_t pack4(uint32_t w)  // 4 int8 -> 2 packed bytes in bits 0..15
+{
+    uint32_t t = w & 0x0F0F0F0Fu;
+    t |= t >> 4;  // byte0 = n0 | n1<<4, byte2 = n2 | n3<<4
+    return (t & 0xFFu) | ((t >> 8) & 0xFF00u);
+}
+
+__global__ void pack_i4_vec_kernel(const v4i *__restrict__ src, v2i *__restrict__ dst, size_t nvec)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (size_t)gridDim.x * blockDim.x) {
+        const v4i v = src[i];
+        v2i o;
+        o.x = (int)(pack4((uint32_t)v.x) | (pack4((uint32_t)v.y) << 16));
+        o.y = (int)(pack4((uint32_t)v.z) | (pack4((uint32_t)v.w) << 16));
+        dst[i] = o;
+    }
+}
+
+__global__ void pack_i4_byte_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, size_t nbytes)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nbytes; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = (uint8_t)((src[2 * i] & 0x0Fu) | ((src[2 * i + 1] & 0x0Fu) << 4));
+}
+
+// 4 packed bytes -> 8 int8: widen nibbles to bytes, sign-extend (bit 3 set => OR 0xF0),
+// interleave even/odd elements back into K order.
+__device__ __forceinline__ uint32_t sext_nibbles(uint32_t x)  // x = 0x0n0n0n0n
+{
+    const uint32_t t = x & 0x08080808u;
+    return x | ((t << 5) - (t << 1));  // 0x08 -> 0xF0 in each byte (the top byte wraps mod 2^32)
+}
+
+__global__ void unpack_i4_vec_kernel(const uint32_t *__restrict__ src, v2i *__restrict__ dst, size_t nwords)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nwords; i += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t w = src[i];
+        const uint32_t ev = sext_nibbles(w & 0x0F0F0F0Fu), od = sext_nibbles((w >> 4) & 0x0F0F0F0Fu);
+        v2i o;  // bytes: ev0 od0 ev1 od1 | ev2 od2 ev3 od3
+        o.x = (int)__builtin_amdgcn_perm(od, ev, 0x05010400u);
+        o.y = (int)__builtin_amdgcn_perm(od, ev, 0x07030602u);
+        dst[i] = o;
+    }
+}
+
+__global__ void unpack_i4_byte_kernel(const uint8_t *__restrict__ src, int8_t *__restrict__ dst, size_t nbytes)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nbytes; i += (size_t)gridDim.x * blockDim.x) {
+        const uint32_t b = src[i];
+        dst[2 * i] = (int8_t)s4_lo(b);
+        dst[2 * i + 1] = (int8_t)s4_hi(b);
+    }
+}
+
+static unsigned flat_grid(size_t items, unsigned block)
+{
+    size_t g = (items + block - 1) / block;
+    if (g < 1) g = 1;
+    if (g > 256u * 32u) g = 256u * 32u;
+    return (unsigned)g;
+}
+
+// --------------------------------------------------------------------------
+// Skinny launchers
+// --------------------------------------------------------------------------
+template <class Cfg>
+static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
+{
+    const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
+    gemm_skinny_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), 0, stream>>>(p);
+    return hipGetLastError();
+}
+#define QM_SKINNY(FM, FN, NW, U) \
+    hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U>>(p, s, gm); }
+#include "qm_configs.inc"
+
+// --------------------------------------------------------------------------
+// Configuration registry
+// --------------------------------------------------------------------------
+enum Kind { KIND_GENERIC = 0, KIND_TILE = 1, KIND_SKINNY = 2 };
+
+struct ConfigDesc {
+    const char *name;
+    int kind;
+    int bm, bn, bk;  // tile: block shape; skinny: bm = max M, bn = columns per workgroup
+    int waves, mode;
+    LaunchFn launch;
+};
+
+#define QM_STR2(x) #x
+#define QM_STR(x) QM_STR2(x)
+static const ConfigDesc g_configs[] = {
+    {"generic", KIND_GENERIC, 16, 16, 128, 4, 0, &launch_generic},
+#define QM_TILE(tu, BM, BN, BK, WGM, WGN, MODE)                                                        \
+    {"t" QM_STR(BM) "x" QM_STR(BN) "x" QM_STR(BK) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_m" QM_STR(MODE), \
+     KIND_TILE, BM, BN, BK, (WGM) * (WGN), MODE, &QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)},
+#define QM_SKINNY(FM, FN, NW, U)                                                     \
+    {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
+     &QM_SKINNY_FN(FM, FN, NW, U)},
+#include "qm_configs.inc"
+};
+static constexpr int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
+
+static int find_config(const char *name)
+{
+    for (int i = 0; i < g_num_configs; ++i)
+        if (std::strcmp(g_configs[i].name, name) == 0) return i;
+    return -1;
+}
+
+// The 16-byte-load kernels need whole, aligned chunks and 32-bit row offsets,
+// and the x16 widening bounds K.
+static bool fast_path_ok(int m, int n, int k, int ptr_align)
+{
+    if (k % 32 != 0 || k > QM_MAX_K_X16 || ptr_align < 16) return false;
+    const long long kb = k / 2;
+    return (long long)m * kb < 0x7fffffffLL && (long long)n * kb < 0x7fffffffLL;
+}
+
+static bool config_supports(int cfg, int m, int n, int k, int ptr_align)
+{
+    if (cfg < 0 || cfg >= g_num_configs || m < 1 || n < 1 || k < 2 || (k & 1)) return false;
+    const ConfigDesc &c = g_configs[cfg];
+    if (c.kind == KIND_GENERIC) return true;
+    if (!fast_path_ok(m, n, k, ptr_align)) return false;
+    if (c.kind == KIND_SKINNY) return m <= c.bm;
+    return true;
+}
+
+// --------------------------------------------------------------------------
+// Shape table (autotuned on MI355X; regenerated by quadmul_amd/autotune.py) with
+// a cost-model fallback -- the reference instead skips unknown shapes.
+// --------------------------------------------------------------------------
+struct TableEntry {
+    int m, n, k;
+    const char *config;
+    int group_m;
+};
+static const TableEntry g_table[] = {
+#include "qm_tile_table.inc"
+    {0, 0, 0, nullptr, 0},
+};
+
+struct Choice {
+    int cfg, group_m;
+};
+
+static Choice heuristic(int m, int n, int k, int ptr_align)
+{
+    if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1};
+    if (m <= 64) {
+        const int fm = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
+        const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w8_u2");
+        const int id = find_config(name);
+        if (id >= 0) return {id, 1};
+    }
+    // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency).
+    static const struct { const char *name; double eff; } cands[] = {
+        {"t256x256x128_w2x2_m0", 1.00}, {"t128x256x128_w2x2_m0", 0.88}, {"t256x128x128_w2x2_m0", 0.88},
+        {"t128x128x128_w2x2_m0", 0.72}, {"t64x256x128_w1x4_m0", 0.62},  {"t64x128x128_w2x2_m0", 0.50},
+        {"t128x64x128_w2x2_m0", 0.50},  {"t64x64x128_w2x2_m0", 0.33},
+    };
+    int best = 0;
+    double best_cost = 1e300;
+    for (const auto &c : cands) {
+        const int id = find_config(c.name);
+        if (id < 0) continue;
+        const ConfigDesc &d = g_configs[id];
+        const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
+        const long long rounds = (tiles + 255) / 256;
+        const double cost = (double)rounds * d.bm * d.bn / c.eff;
+        if (cost < best_cost) { best_cost = cost; best = id; }
+    }
+    return {best, 4};
+}
+
+static Choice select_config(int m, int n, int k, int ptr_align)
+{
+    static int resolved[sizeof(g_table) / sizeof(g_table[0])];
+    static std::once_flag once;
+    std::call_once(once, [] {
+        for (size_t i = 0; g_table[i].config; ++i) resolved[i] = find_config(g_table[i].config);
+    });
+    for (size_t i = 0; g_table[i].config; ++i)
+        if (g_table[i].m == m && g_table[i].n == n && g_table[i].k == k && resolved[i] >= 0 &&
+            config_supports(resolved[i], m, n, k, ptr_align))
+            return {resolved[i], g_table[i].group_m};
+    return heuristic(m, n, k, ptr_align);
+}
+
+static thread_local int g_last_hip_error = 0;
+
+static int ptr_alignment(const void *a, const void *b)
+{
+    const uintptr_t x = (uintptr_t)a | (uintptr_t)b;
+    if (x == 0) return 4096;
+    const uintptr_t low = x & (~x + 1);
+    return low > 4096 ? 4096 : (int)low;
+}
+
+static int check_gemm_args(const void *A, const void *B, void *C, int m, int n, int k)
+{
+    if (m < 0 || n < 0 || k < 0 || (k & 1)) return QM_ERR_SHAPE;
+    if (m == 0 || n == 0) return QM_OK;
+    if (!C) return QM_ERR_NULL;
+    if ((uintptr_t)C & 3) return QM_ERR_ALIGN;
+    if (k > 0 && (!A || !B)) return QM_ERR_NULL;
+    return QM_OK;
+}
+
+static int fail_launch(hipError_t e)
+{
+    g_last_hip_error = (int)e;
+    return QM_ERR_LAUNCH;
+}
+
+}  // namespace qm
+
+using namespace qm;
+
+QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg)
+{
+    const int st = check_gemm_args(A, B, C, m, n, k);
+    if (st != QM_OK) return st;
+    if (m == 0 || n == 0) return QM_OK;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (k == 0) {
+        const size_t cnt = (size_t)m * (size_t)n;
+        fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(C), cnt);
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? QM_OK : fail_launch(e);
+    }
+    const int align = ptr_alignment(A, B);
+    Choice ch;
+    if (cfg == QM_CFG_AUTO) {
+        ch = select_config(m, n, k, align);
+    } else {
+        ch.cfg = cfg & 0xFFFF;
+        ch.group_m = (cfg >> 16) & 0xFF;
+        if (ch.group_m == 0) ch.group_m = 4;
+        if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
+    }
+    const GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(C), m, n, k};
+    const hipError_t e = g_configs[ch.cfg].launch(p, s, ch.group_m);
+    return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
+QM_EXPORT int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, int k, void *stream)
+{
+    return qm_gemm_i4_cfg(A, B, C, m, n, k, stream, QM_CFG_AUTO);
+}
+
+QM_EXPORT int qm_select_config(int m, int n, int k, int ptr_align)
+{
+    if (m < 1 || n < 1 || k < 2 || (k & 1)) return QM_ERR_SHAPE;
+    const Choice ch = select_config(m, n, k, ptr_align);
+    return ch.cfg | (ch.group_m << 16);
+}
+
+QM_EXPORT int qm_num_configs(void) { return g_num_configs; }
+
+QM_EXPORT const char *qm_config_name(int cfg)
+{
+    cfg &= 0xFFFF;
+    return (cfg >= 0 && cfg < g_num_configs) ? g_configs[cfg].name : nullptr;
+}
+
+QM_EXPORT int qm_config_supports(int cfg, int m, int n, int k, int ptr_align)
+{
+    return config_supports(cfg & 0xFFFF, m, n, k, ptr_align) ? 1 : 0;
+}
+
+QM_EXPORT int qm_pack_i4(const void *src_i8, void *dst_packed, int rows, int k, void *stream)
+{
+    if (rows < 0 || k < 0 || (k & 1)) return QM_ERR_SHAPE;
+    const size_t nbytes = (size_t)rows * (size_t)(k / 2);
+    if (nbytes == 0) return QM_OK;
+    if (!src_i8 || !dst_packed) return QM_ERR_NULL;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (nbytes % 8 == 0 && ((uintptr_t)src_i8 & 15) == 0 && ((uintptr_t)dst_packed & 7) == 0)
+        pack_i4_vec_kernel<<<dim3(flat_grid(nbytes / 8, 256)), dim3(256), 0, s>>>(static_cast<const v4i *>(src_i8), static_cast<v2i *>(dst_packed), nbytes / 8);
+    else
+        pack_i4_byte_kernel<<<dim3(flat_grid(nbytes, 256)), dim3(256), 0, s>>>(static_cast<const uint8_t *>(src_i8), static_cast<uint8_t *>(dst_packed), nbytes);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
+QM_EXPORT int qm_unpack_i4(const void *src_packed, void *dst_i8, int rows, int k, void *stream)
+{
+    if (rows < 0 || k < 0 || (k & 1)) return QM_ERR_SHAPE;
+    const size_t nbytes = (size_t)rows * (size_t)(k / 2);
+    if (nbytes == 0) return QM_OK;
+    if (!src_packed || !dst_i8) return QM_ERR_NULL;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (nbytes % 4 == 0 && ((uintptr_t)src_packed & 3) == 0 && ((uintptr_t)dst_i8 & 7) == 0)
+        unpack_i4_vec_kernel<<<dim3(flat_grid(nbytes / 4, 256)), dim3(256), 0, s>>>(static_cast<const uint32_t *>(src_packed), static_cast<v2i *>(dst_i8), nbytes / 4);
+    else
+        unpack_i4_byte_kernel<<<dim3(flat_grid(nbytes, 256)), dim3(256), 0, s>>>(static_cast<const uint8_t *>(src_packed), static_cast<int8_t *>(dst_i8), nbytes);
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
+QM_EXPORT const char *qm_status_string(int status)
+{
+    switch (status) {
+    case QM_OK: return "ok";
+    case QM_ERR_NULL: return "null pointer";
+    case QM_ERR_SHAPE: return "bad shape (m, n, k must be >= 0 and k even)";
+    case QM_ERR_CONFIG: return "unknown kernel configuration, or it cannot run this shape";
+    case QM_ERR_LAUNCH: return "HIP launch failed";
+    case QM_ERR_ALIGN: return "C must be 4-byte aligned";
+    default: return "unknown status";
+    }
+}
+
+QM_EXPORT int qm_last_hip_error(void) { return g_last_hip_error; }
+
+QM_EXPORT const char *qm_version(void) { return "quadmul-amd 0.1 (gfx950)"; }

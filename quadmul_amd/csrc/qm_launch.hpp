@@ -1,0 +1,37 @@
+// Host-side launch plumbing shared by the translation units of libqm_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "qm_common.hpp"
+
+namespace qm {
+
+// Launchers return hipSuccess or the error of the failed runtime call.
+typedef hipError_t (*LaunchFn)(const GemmArgs &, hipStream_t, int group_m);
+
+constexpr int QM_MAX_DEVICES = 64;
+
+// Kernels that want more than 64 KiB of dynamic LDS must say so once per device.
+template <class KernelPtr>
+inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, bool *done_per_device)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= QM_MAX_DEVICES) return hipErrorInvalidDevice;
+    if (!done_per_device[dev]) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return e;
+        done_per_device[dev] = true;
+    }
+    return hipSuccess;
+}
+
+#define QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE) qm_launch_tile_##BM##_##BN##_##BK##_##WGM##_##WGN##_##MODE
+#define QM_SKINNY_FN(FM, FN, NW, U) qm_launch_skinny_##FM##_##FN##_##NW##_##U
+
+#define QM_TILE(tu, BM, BN, BK, WGM, WGN, MODE) \
+    hipError_t QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)(const GemmArgs &, hipStream_t, int);
+#define QM_SKINNY(FM, FN, NW, U) hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &, hipStream_t, int);
+#include "qm_configs.inc"
+
+}  // namespace qm

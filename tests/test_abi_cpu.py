@@ -1,0 +1,103 @@
+"""No-GPU checks of the C-ABI library and the host-side interface: the library
+loads, exports every symbol include/qm_abi.h declares, rejects bad arguments with
+the documented status codes, and selects sensible configurations.  No kernel is
+launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import quadmul_amd as qm
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "qm_abi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(qm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = qm.library()
+    syms = declared_symbols()
+    assert set(syms) == set(qm.ABI_SYMBOLS)
+    for s in syms:
+        assert hasattr(lib, s), s
+
+
+def test_extension_module_imports_and_mirrors_reference_entry_point():
+    import quadmul  # the drop-in module name (setup.py:8,11 of the reference)
+
+    assert callable(quadmul.gemm)
+    assert "Int4xInt4 Matrix Multiplication Kernel" in quadmul.gemm.__doc__  # extension.cpp:28
+    assert quadmul.num_configs() == qm.num_configs()
+
+
+def test_status_codes_without_a_gpu():
+    lib = qm.library()
+    one = ctypes.c_void_p(4096)  # never dereferenced: the checks come first
+    assert lib.qm_gemm_i4(one, one, one, 4, 4, 3, None) == -2      # odd k
+    assert lib.qm_gemm_i4(one, one, one, -1, 4, 4, None) == -2     # negative m
+    assert lib.qm_gemm_i4(None, one, one, 4, 4, 4, None) == -1     # null A
+    assert lib.qm_gemm_i4(one, one, None, 4, 4, 4, None) == -1     # null C
+    assert lib.qm_gemm_i4(one, one, ctypes.c_void_p(4098), 4, 4, 4, None) == -5
+    assert lib.qm_gemm_i4(None, None, None, 0, 4, 4, None) == 0    # empty: nothing to do
+    assert lib.qm_gemm_i4(None, None, None, 4, 0, 4, None) == 0
+    assert lib.qm_gemm_i4_cfg(one, one, one, 4, 4, 4, None, 9999) == -3
+    assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("t128x128x128_w2x2_m0")) == -3
+    assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
+    assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
+    assert lib.qm_unpack_i4(None, one, 4, 8, None) == -1
+    for code in (0, -1, -2, -3, -4, -5):
+        assert lib.qm_status_string(code)
+    assert b"gfx950" in lib.qm_version()
+
+
+def test_config_registry():
+    names = qm.config_names()
+    assert names[0] == "generic" and len(names) == len(set(names))
+    assert any(n.startswith("t256x256") for n in names) and any(n.startswith("s1x1") for n in names)
+    for i, n in enumerate(names):
+        assert qm.config_id(n) == i
+    with pytest.raises(qm.QuadmulError):
+        qm.config_name(len(names))
+
+
+def test_selection_rules():
+    name = lambda m, n, k, al=256: qm.config_name(qm.select_config(m, n, k, al) & 0xFFFF)
+    assert name(8192, 8192, 8192).startswith("t")
+    assert name(4096, 4096, 4096).startswith("t")
+    for m in (1, 16, 64):
+        assert name(m, 4096, 4096).startswith("s"), m
+    assert name(100, 100, 30) == "generic"          # K % 32 != 0: no 16-byte chunks
+    assert name(128, 128, 4096, 4) == "generic"     # operands not 16-byte aligned
+    assert name(128, 128, 262144) == "generic"      # beyond the exact range of the x16 widening
+    gid, sk = qm.config_id("generic"), qm.config_id("s1x1_w8_u4")
+    assert qm.config_supports(gid, 3, 5, 2, 1)
+    assert qm.config_supports(sk, 16, 4096, 4096) and not qm.config_supports(sk, 17, 4096, 4096)
+    assert not qm.config_supports(sk, 16, 4096, 4098)
+
+
+def test_host_checks_reject_bad_tensors():
+    a = torch.zeros(4, 4, dtype=torch.int8)
+    c = torch.zeros(4, 4, dtype=torch.int32)
+    with pytest.raises(qm.QuadmulError):
+        qm.gemm(a, a, c, 4, 4, 8)  # CPU tensors
+    import quadmul
+    with pytest.raises(RuntimeError):
+        quadmul.gemm(a, a, c, 4, 4, 8)
+
+
+def test_cpu_pack_unpack_mirror_reference_semantics():
+    from util import make_values, pack_cpu
+
+    v = make_values(9, 64, 3)
+    p = qm.pack_int4(v)
+    assert p.dtype == torch.int8 and p.shape == (9, 32)
+    assert torch.equal(p, pack_cpu(v))
+    assert torch.equal(qm.unpack_int4(p), v)
+    with pytest.raises(qm.QuadmulError):
+        qm.pack_int4(torch.zeros(2, 3, dtype=torch.int8))

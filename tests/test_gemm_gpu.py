@@ -1,0 +1,245 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle --
+bit-exact, on seeded inputs, with C pre-poisoned to prove it is overwritten."""
+import numpy as np
+import pytest
+import torch
+
+import quadmul_amd as qm
+from util import SEED_BASE, make_operands, pack_cpu, poisoned_c
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def run_gemm(ap, bp, m, n, k, cfg=qm.CFG_AUTO):
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    c_d = poisoned_c(m, n, DEV)
+    qm.gemm_cfg(a_d, b_d, c_d, m, n, k, cfg)
+    torch.cuda.synchronize()
+    return c_d.cpu().numpy()
+
+
+def fp32_matmul_on_gpu(a, b):
+    """Exact for these sizes: every partial sum is an integer below 2^24."""
+    a_d, b_d = a.to(DEV).float(), b.to(DEV).float()
+    out = torch.empty((a.shape[0], b.shape[0]), dtype=torch.int32, device=DEV)
+    for i in range(0, a.shape[0], 2048):
+        out[i:i + 2048] = (a_d[i:i + 2048] @ b_d.t()).to(torch.int32)
+    return out
+
+
+SMALL_SHAPES = [
+    (1, 1, 32), (1, 16, 64), (2, 15, 96), (15, 17, 128), (16, 16, 160), (17, 63, 256), (33, 65, 224),
+    (63, 130, 512), (64, 64, 1024), (65, 255, 384), (127, 129, 640), (128, 256, 4096), (200, 300, 1184),
+    (256, 256, 128), (257, 511, 288), (300, 70, 2080),
+]
+
+
+@pytest.mark.parametrize("shape", SMALL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_every_config_matches_oracle(oracle_mod, shape):
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 1000 + m * 7 + n * 3 + k)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    ran = 0
+    for cfg, name in enumerate(qm.config_names()):
+        if not qm.config_supports(cfg, m, n, k):
+            continue
+        for gm in (1, 3):
+            got = run_gemm(ap, bp, m, n, k, cfg | (gm << 16))
+            bad = oracle_mod.compare(got, want)
+            assert bad == -1, f"{name} group_m={gm}: first mismatch at flat index {bad}: got {got.flat[bad]} want {want.flat[bad]}"
+        ran += 1
+    assert ran >= 2
+    got = run_gemm(ap, bp, m, n, k)
+    assert oracle_mod.compare(got, want) == -1
+
+
+GENERIC_SHAPES = [(1, 1, 2), (3, 5, 30), (17, 33, 34), (70, 33, 160 + 2), (100, 130, 510), (5, 130, 34)]
+
+
+@pytest.mark.parametrize("shape", GENERIC_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_k_not_multiple_of_32_takes_generic_path(oracle_mod, shape):
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 2000 + k)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    assert qm.config_name(qm.select_config(m, n, k) & 0xFFFF) == "generic"
+    assert oracle_mod.compare(run_gemm(ap, bp, m, n, k), oracle_mod.gemm_i4(ap.numpy(), bp.numpy())) == -1
+
+
+def test_unaligned_operands_take_generic_path(oracle_mod):
+    m, n, k = 37, 41, 128
+    a, b = make_operands(m, n, k, SEED_BASE + 2100)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    buf_a = torch.zeros(ap.numel() + 16, dtype=torch.int8, device=DEV)
+    buf_b = torch.zeros(bp.numel() + 16, dtype=torch.int8, device=DEV)
+    a_d = buf_a[3:3 + ap.numel()].view(m, k // 2)
+    b_d = buf_b[5:5 + bp.numel()].view(n, k // 2)
+    a_d.copy_(ap)
+    b_d.copy_(bp)
+    c_d = poisoned_c(m, n, DEV)
+    qm.gemm(a_d, b_d, c_d, m, n, k)
+    assert oracle_mod.compare(c_d.cpu().numpy(), oracle_mod.gemm_i4(ap.numpy(), bp.numpy())) == -1
+
+
+@pytest.mark.parametrize("name", ["gemm_i4_32x48x64", "gemm_i4_70x33x160", "gemm_i4_5x130x34"])
+def test_golden_fixtures(name):
+    import os
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", name + ".npz"))
+    m, k = z["a"].shape
+    n = z["b"].shape[0]
+    got = run_gemm(torch.from_numpy(z["a_packed"]), torch.from_numpy(z["b_packed"]), m, n, k)
+    assert (got == z["c"]).all()
+
+
+def test_nibble_product_table_and_one_hot(oracle_mod):
+    s4 = lambda v: v - 16 if v > 7 else v
+    vals = torch.tensor([s4(i) for i in range(16)], dtype=torch.int8)
+    k = 64
+    for pos in (0, 1, 30, 31, 32, 33, 63):
+        a = torch.zeros(16, k, dtype=torch.int8)
+        a[:, pos] = vals
+        got = run_gemm(pack_cpu(a), pack_cpu(a), 16, 16, k)
+        assert (got == np.outer(vals.numpy().astype(np.int32), vals.numpy().astype(np.int32))).all(), pos
+        b = torch.zeros(16, k, dtype=torch.int8)
+        b[:, pos ^ 1] = vals
+        assert (run_gemm(pack_cpu(a), pack_cpu(b), 16, 16, k) == 0).all(), pos
+
+
+@pytest.mark.parametrize("shape", [(16, 64, 4096), (80, 272, 11008), (300, 260, 28672)], ids=lambda s: "x".join(map(str, s)))
+def test_extremes_closed_form_on_every_config(shape):
+    m, n, k = shape
+    lo_a = pack_cpu(torch.full((m, k), -8, dtype=torch.int8))
+    lo_b = pack_cpu(torch.full((n, k), -8, dtype=torch.int8))
+    hi_b = pack_cpu(torch.full((n, k), 7, dtype=torch.int8))
+    for cfg, name in enumerate(qm.config_names()):
+        if not qm.config_supports(cfg, m, n, k) or name == "generic":
+            continue
+        assert (run_gemm(lo_a, lo_b, m, n, k, cfg) == 64 * k).all(), name   # largest positive accumulator
+        assert (run_gemm(lo_a, hi_b, m, n, k, cfg) == -56 * k).all(), name  # most negative accumulator
+
+
+def test_largest_exact_k_and_beyond(oracle_mod):
+    # K = 131040 is the largest multiple of 32 the x16 widening covers exactly; past it the
+    # generic kernel must take over, with the same results.
+    m, n = 16, 32
+    for k in (131040, 131072):
+        a = pack_cpu(torch.full((m, k), -8, dtype=torch.int8))
+        b = pack_cpu(torch.full((n, k), -8, dtype=torch.int8))
+        assert (run_gemm(a, b, m, n, k) == 64 * k).all(), k
+    assert qm.config_name(qm.select_config(m, n, 131072) & 0xFFFF) == "generic"
+
+
+def test_dtypes_and_overwrite(oracle_mod):
+    m, n, k = 48, 80, 256
+    a, b = make_operands(m, n, k, SEED_BASE + 3000)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    for view in (torch.int8, torch.uint8):
+        a_d, b_d = ap.to(DEV).view(view), bp.to(DEV).view(view)
+        c_d = poisoned_c(m, n, DEV)
+        qm.gemm(a_d, b_d, c_d, m, n, k)
+        assert oracle_mod.compare(c_d.cpu().numpy(), want) == -1
+        qm.gemm(a_d, b_d, c_d, m, n, k)  # twice into the same C: overwrite, not accumulate
+        assert oracle_mod.compare(c_d.cpu().numpy(), want) == -1
+
+
+def test_k_zero_and_empty():
+    c = poisoned_c(5, 7, DEV)
+    e = torch.empty((5, 0), dtype=torch.int8, device=DEV)
+    qm.gemm(e, torch.empty((7, 0), dtype=torch.int8, device=DEV), c, 5, 7, 0)
+    assert (c == 0).all()
+    qm.gemm(torch.empty((0, 16), dtype=torch.int8, device=DEV), torch.empty((7, 16), dtype=torch.int8, device=DEV),
+            torch.empty((0, 7), dtype=torch.int32, device=DEV), 0, 7, 32)
+
+
+def test_extension_module_runs_on_side_stream_and_under_graph_replay(oracle_mod):
+    import quadmul
+
+    m, n, k = 96, 160, 512
+    a, b = make_operands(m, n, k, SEED_BASE + 3100)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    c_d = poisoned_c(m, n, DEV)
+    quadmul.gemm(a_d, b_d, c_d, m, n, k)  # positional, as test.py:40
+    torch.cuda.synchronize()
+    assert oracle_mod.compare(c_d.cpu().numpy(), want) == -1
+
+    side = torch.cuda.Stream()
+    c2 = poisoned_c(m, n, DEV)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        quadmul.gemm(a_d, b_d, c2, m, n, k)
+    side.synchronize()
+    assert oracle_mod.compare(c2.cpu().numpy(), want) == -1
+
+    # captured as the reference's harness does (test.py:78-81); every replay is checked
+    c3 = poisoned_c(m, n, DEV)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(3):
+            quadmul.gemm(a_d, b_d, c3, m, n, k)
+    for _ in range(3):
+        c3.fill_(0x7F7F7F7F)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert oracle_mod.compare(c3.cpu().numpy(), want) == -1
+
+
+def test_pack_unpack_kernels(oracle_mod):
+    from util import make_values
+
+    for rows, k in [(1, 2), (3, 6), (7, 30), (16, 64), (33, 130), (128, 4096), (257, 1184)]:
+        v = make_values(rows, k, SEED_BASE + 4000 + rows)
+        want_p = oracle_mod.pack_i4(v.numpy())
+        got_p = qm.pack_int4(v.to(DEV))
+        assert (got_p.cpu().numpy().view(np.uint8) == want_p).all(), (rows, k)
+        got_u = qm.unpack_int4(got_p)
+        assert (got_u.cpu().numpy() == oracle_mod.unpack_i4(want_p)).all(), (rows, k)
+        assert torch.equal(got_u.cpu(), v)
+    allb = torch.arange(256, dtype=torch.uint8).view(4, 64).to(DEV)
+    assert (qm.unpack_int4(allb).cpu().numpy() == oracle_mod.unpack_i4(allb.cpu().numpy())).all()
+    assert torch.equal(qm.pack_int4(qm.unpack_int4(allb)).view(torch.uint8), allb)
+
+
+# ------------------------------------------------------------------ the named workloads
+BASELINE_SHAPES = [
+    (0, 1024, 1024, 1024), (1, 4096, 4096, 4096),
+    (2, 1, 4096, 4096), (3, 16, 4096, 4096), (4, 64, 4096, 4096),
+    (5, 2048, 11008, 4096), (6, 2048, 4096, 11008), (7, 2048, 12288, 4096),
+]
+
+
+@pytest.mark.parametrize("row", BASELINE_SHAPES, ids=lambda r: "x".join(map(str, r[1:])))
+def test_baseline_configs_full_compare(oracle_mod, row):
+    i, m, n, k = row
+    a, b = make_operands(m, n, k, SEED_BASE + i)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    got_d = poisoned_c(m, n, DEV)
+    qm.gemm(ap.to(DEV), bp.to(DEV), got_d, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.equal(got_d, fp32_matmul_on_gpu(a, b))
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy(), threads=0)
+    assert oracle_mod.compare(got_d.cpu().numpy(), want) == -1
+
+
+@pytest.mark.parametrize("row", [(8, 8192, 8192, 8192), (9, 8000, 8000, 8064)], ids=lambda r: "x".join(map(str, r[1:])))
+def test_large_configs(oracle_mod, row):
+    i, m, n, k = row
+    a, b = make_operands(m, n, k, SEED_BASE + i)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    got_d = poisoned_c(m, n, DEV)
+    qm.gemm(ap.to(DEV), bp.to(DEV), got_d, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.equal(got_d, fp32_matmul_on_gpu(a, b))  # every element
+    rows = np.unique(np.concatenate([np.arange(0, m, 97), [m - 1, m - 2, 255, 256, 257]])).astype(np.int32)
+    want = oracle_mod.gemm_i4_rows(ap.numpy(), bp.numpy(), rows)
+    got = got_d.cpu().numpy()[rows]
+    assert oracle_mod.compare(got, want) == -1
+    # a checksum the layout cannot fake: column sums of C equal (sum of A rows) . B^T
+    colsum = a.to(torch.int64).sum(0)
+    want_cs = (b.to(torch.int64) * colsum).sum(1)
+    assert torch.equal(got_d.to(torch.int64).sum(0).cpu(), want_cs)
