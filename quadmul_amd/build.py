@@ -28,13 +28,13 @@ CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 OBJDIR = os.path.join(PKG, "build")
 LIB_PATH = os.path.join(LIBDIR, "libqm_hip.so")
-N_TILE_TUS = 8
+N_TILE_TUS = 16
 
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm", "-I", os.path.join(ROOT, "include"), "-I", CSRC,
 ]
 
 

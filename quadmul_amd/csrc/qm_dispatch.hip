@@ -145,7 +145,7 @@ static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
 // --------------------------------------------------------------------------
 // Configuration registry
 // --------------------------------------------------------------------------
-enum Kind { KIND_GENERIC = 0, KIND_TILE = 1, KIND_SKINNY = 2 };
+enum Kind { KIND_GENERIC = 0, KIND_TILE = 1, KIND_SKINNY = 2, KIND_TILE32 = 3, KIND_TILE16 = 4 };
 
 struct ConfigDesc {
     const char *name;
@@ -162,6 +162,12 @@ static const ConfigDesc g_configs[] = {
 #define QM_TILE(tu, BM, BN, BK, WGM, WGN, MODE)                                                        \
     {"t" QM_STR(BM) "x" QM_STR(BN) "x" QM_STR(BK) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_m" QM_STR(MODE), \
      KIND_TILE, BM, BN, BK, (WGM) * (WGN), MODE, &QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)},
+#define QM_TILE32(tu, BM, BN, WGM, WGN)                                                              \
+    {"p" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN), KIND_TILE32, BM, BN, 128, (WGM) * (WGN), 0, \
+     &QM_TILE32_FN(BM, BN, WGM, WGN)},
+#define QM_TILE16(tu, BM, BN, WGM, WGN)                                                              \
+    {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN), KIND_TILE16, BM, BN, 128, (WGM) * (WGN), 0, \
+     &QM_TILE16_FN(BM, BN, WGM, WGN)},
 #define QM_SKINNY(FM, FN, NW, U)                                                     \
     {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
      &QM_SKINNY_FN(FM, FN, NW, U)},
@@ -192,6 +198,7 @@ static bool config_supports(int cfg, int m, int n, int k, int ptr_align)
     if (c.kind == KIND_GENERIC) return true;
     if (!fast_path_ok(m, n, k, ptr_align)) return false;
     if (c.kind == KIND_SKINNY) return m <= c.bm;
+    if (c.kind == KIND_TILE32 || c.kind == KIND_TILE16) return k % 128 == 0;  // whole K-steps only: its loop has no tail path
     return true;
 }
 

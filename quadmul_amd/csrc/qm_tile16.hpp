@@ -1,0 +1,270 @@
+// Software-pipelined int4 GEMM tile kernel on v_mfma_i32_16x16x64_i8 (gfx950).
+//
+// Takes the place of the reference's igemm<Config> (kernel.cu:62-266) for large
+// tiles: its cp.async loaders (kernel.cu:118-152) become direct global->LDS loads,
+// its two-stage pipeline (kernel.cu:186-260) a four-stage LDS ring, its WMMA s4
+// contraction (kernel.cu:246) int8 MFMAs on nibbles widened to 16*s4.
+//
+// What shapes it (all measured on MI355X):
+//   * The part runs this workload at its package power limit, so energy spent
+//     outside the MFMAs costs throughput directly.  Under the power cap the
+//     16x16x64 int8 MFMA sustains a clearly higher rate than the 32x32x32 one, and
+//     operands of the form 16*s4 (low nibble zero) are cheaper than sign-extended.
+//   * LDS holds the packed bytes (half the LDS traffic of an int8 tile); each wave
+//     widens its own fragments after ds_read: 3 VALU instructions per dword.
+//   * Tiles travel global -> LDS without touching registers (global_load_lds, 16
+//     bytes per lane): no staging registers, no ds_write.  Ring of 4 stages: while
+//     tile t is contracted, B fragments of tile t+1 are read and widened, tile t+2
+//     has landed and tile t+3 is in flight; one barrier per K-step.
+//   * The compiler's scheduler, left alone, puts the two MFMAs that update one
+//     accumulator back to back and bunches the VALU work, which stalls the matrix
+//     pipe.  The K-step is therefore written slot by slot -- one MFMA plus its share
+//     of reads / widening / DMA -- with a scheduling barrier after every slot.
+#pragma once
+#include <type_traits>
+
+#include "qm_common.hpp"
+
+namespace qm {
+
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
+// acc += S0 * S1 with the accumulator pinned in AGPRs and tied in place.  Written as
+// an asm statement for two reasons: the register allocator otherwise shuffles the 256
+// accumulator registers around at the loop back-edge (hundreds of v_accvgpr moves per
+// iteration), and volatile asm statements keep their program order, which is the issue
+// order this kernel is built around.  The compiler cannot see the MFMA inside, so the
+// kernel keeps every producer of S0/S1 and every other user of `acc` several
+// instructions away (no MFMA hazard wait states are needed at those distances).
+__device__ __forceinline__ void mfma16_acc(v4i &acc, const v4i &s0, const v4i &s1)
+{
+    asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(s0), "v"(s1));
+}
+
+template <int BM_, int BN_, int WGM_, int WGN_>
+struct Tile16Cfg {
+    static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_;
+    static constexpr int WAVES = WGM * WGN, THREADS = 64 * WAVES;
+    static constexpr int WM = BM / WGM, WN = BN / WGN;
+    static constexpr int FM = WM / 16, FN = WN / 16;  // 16x16 accumulator blocks per wave
+    static constexpr int PITCH = 64;                  // packed bytes per row per K-step
+    static constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
+    static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static constexpr int STAGES = 4;
+    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+    // one DMA piece = one wave-wide 16-byte-per-lane load = 16 rows x 64 bytes
+    static constexpr int A_PIECES = BM / 16 / WAVES, B_PIECES = BN / 16 / WAVES;
+    static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile is a multiple of 16x16");
+    static_assert(BM % (16 * WAVES) == 0 && BN % (16 * WAVES) == 0, "DMA pieces must divide evenly among the waves");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
+    static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
+    static_assert((12 * FN) % FM == 0, "B widening must split evenly over the sub-steps");
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::THREADS)
+gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const int group_m)
+{
+    constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, FM = Cfg::FM, FN = Cfg::FN;
+    constexpr int PITCH = Cfg::PITCH, STAGE = Cfg::STAGE_BYTES, WAVES = Cfg::WAVES;
+    constexpr int A_PIECES = Cfg::A_PIECES, B_PIECES = Cfg::B_PIECES, NP = A_PIECES + B_PIECES;
+
+    extern __shared__ __align__(16) uint8_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / Cfg::WGN, wn = wave % Cfg::WGN;
+    const int r = lane & 15, g = lane >> 4;
+
+    const int pid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int width = group_m * tiles_n;
+    const int first_m = (pid / width) * group_m;
+    const int gsz = min(tiles_m - first_m, group_m);
+    const int m0 = (first_m + (pid % width) % gsz) * BM;
+    const int n0 = ((pid % width) / gsz) * BN;
+
+    const int Kb = p.K >> 1;
+    const int KT = p.K / BK;  // K is a multiple of 128 for this kernel
+
+    // ---- global -> LDS: piece q of this wave covers tile rows (q*WAVES + wave)*16 .. +15.
+    // The hardware puts lane l's 16 bytes at (wave-uniform LDS base) + 16*l, i.e. row l/4,
+    // physical chunk l%4 of the piece; the lane therefore fetches the logical chunk that
+    // the swizzle (chunk ^ ((row >> 1) & 3)) maps there.  Rows past the edge of the matrix
+    // are clamped (their products are never stored).
+    const int dma_row = lane >> 2;
+    const int dma_ch = (lane & 3) ^ ((dma_row >> 1) & 3);
+    uint32_t a_goff[A_PIECES], b_goff[B_PIECES];
+#pragma unroll
+    for (int q = 0; q < A_PIECES; ++q)
+        a_goff[q] = (uint32_t)min(m0 + (q * WAVES + wave) * 16 + dma_row, p.M - 1) * (uint32_t)Kb + dma_ch * 16;
+#pragma unroll
+    for (int q = 0; q < B_PIECES; ++q)
+        b_goff[q] = (uint32_t)min(n0 + (q * WAVES + wave) * 16 + dma_row, p.N - 1) * (uint32_t)Kb + dma_ch * 16;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+    const uint32_t dma_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 16 * PITCH);
+
+    // piece index -> (operand, piece): issues one wave-wide load of tile `kt` into `stage_byte`.
+    // Tiles past the end re-read the last tile; they land in a stage nobody reads any more.
+    auto dma_piece = [&](int piece, int stage_byte, int kt) {
+        const int kofs = min(kt, KT - 1) * (BK / 2);
+        if (piece < A_PIECES) {
+            const uint32_t dst = dma_lds + stage_byte + piece * WAVES * 16 * PITCH;
+            const uint8_t *src = p.A + kofs;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(a_goff[piece]), "s"(src) : "memory", "m0");
+        } else {
+            const int b = piece - A_PIECES;
+            const uint32_t dst = dma_lds + stage_byte + Cfg::A_BYTES + b * WAVES * 16 * PITCH;
+            const uint8_t *src = p.B + kofs;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(b_goff[b]), "s"(src) : "memory", "m0");
+        }
+    };
+
+    // ---- fragment reads: lane -> row r of a 16-row fragment, chunk g (32 nibbles) ----
+    // (rows of consecutive fragments differ by 16, which leaves (row >> 1) & 3 unchanged)
+    const int a_row = wm * Cfg::WM + r, b_row = wn * Cfg::WN + r;
+    const int a_rd = a_row * PITCH + ((g ^ ((a_row >> 1) & 3)) << 4);
+    const int b_rd = Cfg::A_BYTES + b_row * PITCH + ((g ^ ((b_row >> 1) & 3)) << 4);
+    auto read_a = [&](int stage_byte, int i) -> v4i {
+        return *reinterpret_cast<const v4i *>(smem + stage_byte + a_rd + i * 16 * PITCH);
+    };
+    auto read_b = [&](int stage_byte, int j) -> v4i {
+        return *reinterpret_cast<const v4i *>(smem + stage_byte + b_rd + j * 16 * PITCH);
+    };
+
+    // acc[i][j]: B rows feed MFMA source 0 and A rows source 1, so a lane ends up with
+    // 4 consecutive n for one m -- one 16-byte store into row-major C.
+    v4i acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+
+    // ---- prologue: tiles 0, 1, 2 on their way into stages 0, 1, 2; wait for 0 and 1 ----
+#pragma unroll
+    for (int t = 0; t < 3; ++t)
+#pragma unroll
+        for (int q = 0; q < NP; ++q) dma_piece(q, t * STAGE, t);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NP) : "memory");
+    __syncthreads();
+
+    // B fragments of the current tile (widened) and of the next (being widened); the two
+    // sets swap roles every K-step, so the K loop is unrolled by two.  A: ping-pong per
+    // sub-step (FM is even, so the parity carries over K-steps).
+    v4i b_ev[2][FN], b_od[2][FN], b_pk[2];
+    v4i a_ev[2], a_od[2], a_pk[2];
+#pragma unroll
+    for (int j = 0; j < FN; ++j) x16_expand(read_b(0, j), b_ev[0][j], b_od[0][j]);
+    x16_expand(read_a(0, 0), a_ev[0], a_od[0]);
+    a_pk[1] = read_a(0, 1);
+
+    int cur = 0, nxt = STAGE, lnd = 2 * STAGE, fly = 3 * STAGE;  // byte offsets of the ring stages
+
+    // Widening op k (0..11) of a packed fragment: dword k/3; part 0: shift, 1: mask -> even
+    // nibbles, 2: mask -> odd nibbles.
+    auto widen_op = [&](auto k_, const v4i &pk, v4i &ev, v4i &od, const uint32_t mask) {
+        constexpr int k = decltype(k_)::value, d = k / 3, part = k % 3;
+        if constexpr (part == 0) ev[d] = (int)((uint32_t)pk[d] << 4);
+        else if constexpr (part == 1) ev[d] = (int)((uint32_t)ev[d] & mask);
+        else od[d] = (int)((uint32_t)pk[d] & mask);
+    };
+
+    auto k_step = [&](const int kt, auto bs_tag) {
+        constexpr int bs = decltype(bs_tag)::value;  // B register set holding tile kt
+        constexpr int SLOTS = 2 * FN;                // MFMAs per sub-step
+        constexpr int BSHARE = 12 * FN / FM;         // B widening ops per sub-step
+        constexpr int NOPS = 12 + BSHARE;            // VALU ops per sub-step, spread over slots 1..SLOTS-1
+        // The loop runs K-steps in pairs; when the number of tiles is odd the last step
+        // contracts a tile that does not exist, so its B operand is widened to zero.
+        const uint32_t bmask = kt + 1 < KT ? 0xF0F0F0F0u : 0u;
+        static_for<0, FM>([&](auto i_) {
+            constexpr int i = decltype(i_)::value;
+            constexpr int pa = i & 1;
+            static_for<0, SLOTS>([&](auto s_) {
+                constexpr int s = decltype(s_)::value;
+                // -- the MFMA of this slot: even-nibble K-slice for all j, then the odd one --
+                if constexpr (s < FN) mfma16_acc(acc[i][s], b_ev[bs][s], a_ev[pa]);
+                else mfma16_acc(acc[i][s - FN], b_od[bs][s - FN], a_od[pa]);
+                if constexpr (s == 0) {
+                    // -- LDS reads: B fragments of tile kt+1 whose widening starts in this
+                    //    sub-step, and the A fragment two sub-steps ahead --
+                    static_for<0, FN>([&](auto j_) {
+                        constexpr int j = decltype(j_)::value;
+                        if constexpr ((12 * j) / BSHARE == i) b_pk[j & 1] = read_b(nxt, j);
+                    });
+                    constexpr int i2 = i + 2;
+                    a_pk[pa] = read_a(i2 >= FM ? nxt : cur, i2 % FM);
+                } else {
+                    // -- this slot's share of the widening work: ops [lo, hi) of the sub-step's
+                    //    list: 12 ops for the next A fragment, then BSHARE ops of B(kt+1) --
+                    constexpr int lo = (s - 1) * NOPS / (SLOTS - 1), hi = s * NOPS / (SLOTS - 1);
+                    static_for<lo, hi>([&](auto o_) {
+                        constexpr int o = decltype(o_)::value;
+                        if constexpr (o < 12) {
+                            widen_op(std::integral_constant<int, o>{}, a_pk[pa ^ 1], a_ev[pa ^ 1], a_od[pa ^ 1], 0xF0F0F0F0u);
+                        } else {
+                            constexpr int gop = i * BSHARE + (o - 12);  // index into the K-step's B op list
+                            constexpr int j = gop / 12;
+                            widen_op(std::integral_constant<int, gop % 12>{}, b_pk[j & 1], b_ev[bs ^ 1][j], b_od[bs ^ 1][j], bmask);
+                        }
+                    });
+                }
+                // -- DMA pieces of tile kt+3, one sub-step apart --
+                if constexpr (s == SLOTS - 1) {
+                    static_for<0, NP>([&](auto q_) {
+                        constexpr int q = decltype(q_)::value;
+                        if constexpr (q * FM / NP == i) dma_piece(q, fly, kt + 3);
+                    });
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
+        // Tile kt+2 (issued one K-step ago) must have landed, and every wave must be done
+        // reading stage `cur`, before the roles rotate; tile kt+3 stays in flight.
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NP) : "memory");
+        const int t = cur;
+        cur = nxt;
+        nxt = lnd;
+        lnd = fly;
+        fly = t;
+    };
+
+    for (int kt = 0; kt < KT; kt += 2) {
+        k_step(kt, std::integral_constant<int, 0>{});
+        k_step(kt + 1, std::integral_constant<int, 1>{});
+    }
+    // drain the DMA before the LDS is released; let the last MFMAs retire before their
+    // accumulators are read (the compiler does not know the asm statements were MFMAs)
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: drop the factor 256, guarded 16-byte stores ----
+    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int m = m0 + wm * Cfg::WM + i * 16 + r;
+        if (m >= p.M) continue;
+        int32_t *crow = p.C + (size_t)m * p.N;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int n = n0 + wn * Cfg::WN + j * 16 + g * 4;
+            v4i v = acc[i][j];
+            v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
+            if (vec_ok && n + 3 < p.N) {
+                *reinterpret_cast<v4i *>(crow + n) = v;
+            } else {
+                if (n < p.N) crow[n] = v.x;
+                if (n + 1 < p.N) crow[n + 1] = v.y;
+                if (n + 2 < p.N) crow[n + 2] = v.z;
+                if (n + 3 < p.N) crow[n + 3] = v.w;
+            }
+        }
+    }
+}
+
+}  // namespace qm
