@@ -145,7 +145,7 @@ static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
 // --------------------------------------------------------------------------
 // Configuration registry
 // --------------------------------------------------------------------------
-enum Kind { KIND_GENERIC = 0, KIND_TILE = 1, KIND_SKINNY = 2, KIND_TILE32 = 3, KIND_TILE16 = 4 };
+enum Kind { KIND_GENERIC = 0, KIND_TILE = 1, KIND_SKINNY = 2, KIND_TILE16 = 3 };
 
 struct ConfigDesc {
     const char *name;
@@ -162,9 +162,6 @@ static const ConfigDesc g_configs[] = {
 #define QM_TILE(tu, BM, BN, BK, WGM, WGN, MODE)                                                        \
     {"t" QM_STR(BM) "x" QM_STR(BN) "x" QM_STR(BK) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_m" QM_STR(MODE), \
      KIND_TILE, BM, BN, BK, (WGM) * (WGN), MODE, &QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)},
-#define QM_TILE32(tu, BM, BN, WGM, WGN)                                                              \
-    {"p" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN), KIND_TILE32, BM, BN, 128, (WGM) * (WGN), 0, \
-     &QM_TILE32_FN(BM, BN, WGM, WGN)},
 #define QM_TILE16(tu, BM, BN, WGM, WGN)                                                              \
     {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN), KIND_TILE16, BM, BN, 128, (WGM) * (WGN), 0, \
      &QM_TILE16_FN(BM, BN, WGM, WGN)},
@@ -198,7 +195,7 @@ static bool config_supports(int cfg, int m, int n, int k, int ptr_align)
     if (c.kind == KIND_GENERIC) return true;
     if (!fast_path_ok(m, n, k, ptr_align)) return false;
     if (c.kind == KIND_SKINNY) return m <= c.bm;
-    if (c.kind == KIND_TILE32 || c.kind == KIND_TILE16) return k % 128 == 0;  // whole K-steps only: its loop has no tail path
+    if (c.kind == KIND_TILE16) return k % 128 == 0;  // whole K-steps only: its loop has no tail path
     return true;
 }
 
@@ -229,17 +226,18 @@ static Choice heuristic(int m, int n, int k, int ptr_align)
         const int id = find_config(name);
         if (id >= 0) return {id, 1};
     }
-    // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency).
+    // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency),
+    // over the configurations that can run this K.  Efficiencies are measured ratios.
     static const struct { const char *name; double eff; } cands[] = {
-        {"t256x256x128_w2x2_m0", 1.00}, {"t128x256x128_w2x2_m0", 0.88}, {"t256x128x128_w2x2_m0", 0.88},
-        {"t128x128x128_w2x2_m0", 0.72}, {"t64x256x128_w1x4_m0", 0.62},  {"t64x128x128_w2x2_m0", 0.50},
-        {"t128x64x128_w2x2_m0", 0.50},  {"t64x64x128_w2x2_m0", 0.33},
+        {"q256x256_w2x2", 1.00}, {"q256x128_w2x2", 0.82}, {"q128x256_w2x2", 0.82}, {"q128x128_w2x2", 0.66},
+        {"t256x256x128_w4x2_m0", 0.78}, {"t128x128x128_w2x2_m0", 0.60}, {"t64x128x128_w2x2_m0", 0.40},
+        {"t128x64x128_w2x2_m0", 0.40},  {"t64x64x128_w2x2_m0", 0.30},
     };
     int best = 0;
     double best_cost = 1e300;
     for (const auto &c : cands) {
         const int id = find_config(c.name);
-        if (id < 0) continue;
+        if (id < 0 || !config_supports(id, m, n, k, ptr_align)) continue;
         const ConfigDesc &d = g_configs[id];
         const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
         const long long rounds = (tiles + 255) / 256;

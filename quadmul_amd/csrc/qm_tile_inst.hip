@@ -3,7 +3,6 @@
 #include "qm_launch.hpp"
 #include "qm_tile.hpp"
 #include "qm_tile16.hpp"
-#include "qm_tile32.hpp"
 
 #ifndef QM_TU
 #error "compile with -DQM_TU=<n>"
@@ -18,11 +17,8 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
     hipError_t e = ensure_dynamic_lds(kernel, Cfg::LDS_BYTES, lds_ok);
     if (e != hipSuccess) return e;
     const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
-    const int dbg = group_m & 64;
-    group_m &= 63;
     if (group_m < 1) group_m = 1;
     if (group_m > tiles_m) group_m = tiles_m;
-    group_m |= dbg;
     kernel<<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, tiles_m, tiles_n, group_m);
     return hipGetLastError();
 }
@@ -45,14 +41,6 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
         return launch_tiled<Cfg>(&gemm_tile16_kernel<Cfg>, p, s, gm);                   \
     }                                                                                   \
     }
-#define QM_TILE32_DEF(BM, BN, WGM, WGN)                                                 \
-    namespace qm {                                                                      \
-    hipError_t QM_TILE32_FN(BM, BN, WGM, WGN)(const GemmArgs &p, hipStream_t s, int gm) \
-    {                                                                                   \
-        using Cfg = Tile32Cfg<BM, BN, WGM, WGN>;                                        \
-        return launch_tiled<Cfg>(&gemm_tile32_kernel<Cfg>, p, s, gm);                   \
-    }                                                                                   \
-    }
 
 // An entry of qm_configs.inc is compiled here only when its unit number equals QM_TU:
 // QM_PICK*_<n> expands to nothing except for n == QM_TU.
@@ -68,10 +56,6 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 #define QM_PICK_9(...)
 #define QM_PICK_10(...)
 #define QM_PICK_11(...)
-#define QM_PICK_12(...)
-#define QM_PICK_13(...)
-#define QM_PICK_14(...)
-#define QM_PICK_15(...)
 #define QM_PICK16_0(...)
 #define QM_PICK16_1(...)
 #define QM_PICK16_2(...)
@@ -84,143 +68,70 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 #define QM_PICK16_9(...)
 #define QM_PICK16_10(...)
 #define QM_PICK16_11(...)
-#define QM_PICK16_12(...)
-#define QM_PICK16_13(...)
-#define QM_PICK16_14(...)
-#define QM_PICK16_15(...)
-#define QM_PICK32_0(...)
-#define QM_PICK32_1(...)
-#define QM_PICK32_2(...)
-#define QM_PICK32_3(...)
-#define QM_PICK32_4(...)
-#define QM_PICK32_5(...)
-#define QM_PICK32_6(...)
-#define QM_PICK32_7(...)
-#define QM_PICK32_8(...)
-#define QM_PICK32_9(...)
-#define QM_PICK32_10(...)
-#define QM_PICK32_11(...)
-#define QM_PICK32_12(...)
-#define QM_PICK32_13(...)
-#define QM_PICK32_14(...)
-#define QM_PICK32_15(...)
 #if QM_TU == 0
 #undef QM_PICK_0
 #define QM_PICK_0(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_0
 #define QM_PICK16_0(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_0
-#define QM_PICK32_0(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 1
 #undef QM_PICK_1
 #define QM_PICK_1(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_1
 #define QM_PICK16_1(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_1
-#define QM_PICK32_1(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 2
 #undef QM_PICK_2
 #define QM_PICK_2(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_2
 #define QM_PICK16_2(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_2
-#define QM_PICK32_2(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 3
 #undef QM_PICK_3
 #define QM_PICK_3(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_3
 #define QM_PICK16_3(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_3
-#define QM_PICK32_3(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 4
 #undef QM_PICK_4
 #define QM_PICK_4(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_4
 #define QM_PICK16_4(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_4
-#define QM_PICK32_4(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 5
 #undef QM_PICK_5
 #define QM_PICK_5(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_5
 #define QM_PICK16_5(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_5
-#define QM_PICK32_5(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 6
 #undef QM_PICK_6
 #define QM_PICK_6(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_6
 #define QM_PICK16_6(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_6
-#define QM_PICK32_6(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 7
 #undef QM_PICK_7
 #define QM_PICK_7(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_7
 #define QM_PICK16_7(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_7
-#define QM_PICK32_7(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 8
 #undef QM_PICK_8
 #define QM_PICK_8(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_8
 #define QM_PICK16_8(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_8
-#define QM_PICK32_8(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 9
 #undef QM_PICK_9
 #define QM_PICK_9(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_9
 #define QM_PICK16_9(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_9
-#define QM_PICK32_9(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 10
 #undef QM_PICK_10
 #define QM_PICK_10(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_10
 #define QM_PICK16_10(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_10
-#define QM_PICK32_10(...) QM_TILE32_DEF(__VA_ARGS__)
 #elif QM_TU == 11
 #undef QM_PICK_11
 #define QM_PICK_11(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_11
 #define QM_PICK16_11(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_11
-#define QM_PICK32_11(...) QM_TILE32_DEF(__VA_ARGS__)
-#elif QM_TU == 12
-#undef QM_PICK_12
-#define QM_PICK_12(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_12
-#define QM_PICK16_12(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_12
-#define QM_PICK32_12(...) QM_TILE32_DEF(__VA_ARGS__)
-#elif QM_TU == 13
-#undef QM_PICK_13
-#define QM_PICK_13(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_13
-#define QM_PICK16_13(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_13
-#define QM_PICK32_13(...) QM_TILE32_DEF(__VA_ARGS__)
-#elif QM_TU == 14
-#undef QM_PICK_14
-#define QM_PICK_14(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_14
-#define QM_PICK16_14(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_14
-#define QM_PICK32_14(...) QM_TILE32_DEF(__VA_ARGS__)
-#elif QM_TU == 15
-#undef QM_PICK_15
-#define QM_PICK_15(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_15
-#define QM_PICK16_15(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK32_15
-#define QM_PICK32_15(...) QM_TILE32_DEF(__VA_ARGS__)
 #else
 #error "QM_TU out of range"
 #endif
 
 #define QM_TILE(tu, ...) QM_PICK_##tu(__VA_ARGS__)
 #define QM_TILE16(tu, ...) QM_PICK16_##tu(__VA_ARGS__)
-#define QM_TILE32(tu, ...) QM_PICK32_##tu(__VA_ARGS__)
 #include "qm_configs.inc"

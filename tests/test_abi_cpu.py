@@ -48,6 +48,7 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4(None, None, None, 4, 0, 4, None) == 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 4, 4, 4, None, 9999) == -3
     assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("t128x128x128_w2x2_m0")) == -3
+    assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 160, None, qm.config_id("q256x256_w2x2")) == -3
     assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
     assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
     assert lib.qm_unpack_i4(None, one, 4, 8, None) == -1
@@ -60,6 +61,7 @@ def test_config_registry():
     names = qm.config_names()
     assert names[0] == "generic" and len(names) == len(set(names))
     assert any(n.startswith("t256x256") for n in names) and any(n.startswith("s1x1") for n in names)
+    assert any(n.startswith("q256x256") for n in names)
     for i, n in enumerate(names):
         assert qm.config_id(n) == i
     with pytest.raises(qm.QuadmulError):
@@ -68,8 +70,9 @@ def test_config_registry():
 
 def test_selection_rules():
     name = lambda m, n, k, al=256: qm.config_name(qm.select_config(m, n, k, al) & 0xFFFF)
-    assert name(8192, 8192, 8192).startswith("t")
-    assert name(4096, 4096, 4096).startswith("t")
+    assert name(8192, 8192, 8192).startswith("q")   # pipelined 16x16x64 kernel: K % 128 == 0
+    assert name(4096, 4096, 4096).startswith("q")
+    assert name(4096, 4096, 4096 + 32).startswith("t")  # K % 32 == 0 only: plain tile kernel
     for m in (1, 16, 64):
         assert name(m, 4096, 4096).startswith("s"), m
     assert name(100, 100, 30) == "generic"          # K % 32 != 0: no 16-byte chunks
