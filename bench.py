@@ -128,8 +128,8 @@ def run_workload(name, steps, warmup, check_rows=64):
     fn = lambda: quadmul.gemm(a_d, b_d, c_d, m, n, k)
     fn()
     torch.cuda.synchronize()
+    graph_ms = time_graph(fn)   # also brings the clocks up before the timed steps
     wall_ms, event_ms = time_steps(fn, steps, warmup)
-    graph_ms = time_graph(fn)
     kernel_ms = min(event_ms, graph_ms)
     out = {
         "workload": f"{name}: M={m} N={n} K={k}, signed int4 packed 2/byte along K (low nibble = even k), "
@@ -154,8 +154,10 @@ def cpu_baseline(ap, bp, c_gpu, m, n, k):
     import oracle
 
     threads = oracle.max_threads()
-    rows_mt = min(m, max(16, int(2.0e10 * 1.0 / (n * k))))         # a few seconds of work on all cores
-    rows_1t = min(m, max(4, int(6.0e9 * 1.0 / (n * k))))           # ~1 s on one core
+    # budgets in MACs: about 10 s on all cores, about 10 s on one core (measured rates:
+    # ~1.5e10 MAC/s per core); at 4096^3 the first covers every row of A
+    rows_mt = min(m, max(16, int(1.5e10 * 10 * min(threads, 8) / (n * k))))
+    rows_1t = min(m, max(4, int(1.5e10 * 10 / (n * k))))
     sel_mt = np.linspace(0, m - 1, rows_mt).astype(np.int32)
     t0 = time.perf_counter()
     c_mt = oracle.gemm_i4_rows(ap.numpy(), bp.numpy(), sel_mt, threads=0)
@@ -186,6 +188,11 @@ def main(argv=None):
     ap.add_argument("--workload", default="square4096", choices=sorted(WORKLOADS))
     ap.add_argument("--no-targets", action="store_true", help="skip the other target shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--launches-only", type=int, default=0, metavar="N",
+                    help="profiling aid: just N launches of --workload (after one warm-up), nothing else")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="profiling aid: ten device-to-device copies of 256 MiB (a plain copy kernel of known "
+                         "size, to scale the FETCH_SIZE / WRITE_SIZE counters)")
     a = ap.parse_args(argv)
     if a.gpus != 1:
         print("bench.py: this hot path is a single-GPU kernel and every box here has one GPU; "
@@ -196,6 +203,27 @@ def main(argv=None):
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (no CPU fallback exists for the int4 GEMM)", file=sys.stderr)
         return 2
+
+    if a.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"bytes_read_per_copy": 256 << 20, "bytes_written_per_copy": 256 << 20, "copies": 10}}))
+        return 0
+    if a.launches_only:
+        import quadmul
+
+        row, m, n, k, _ = WORKLOADS[a.workload]
+        apk, bpk = make_packed(m, n, k, SEED_BASE + row)
+        a_d, b_d = apk.to("cuda:0"), bpk.to("cuda:0")
+        c_d = torch.empty((m, n), dtype=torch.int32, device="cuda:0")
+        for _ in range(a.launches_only + 1):
+            quadmul.gemm(a_d, b_d, c_d, m, n, k)
+        torch.cuda.synchronize()
+        print(json.dumps({"launches_only": a.launches_only, "workload": a.workload}))
+        return 0
 
     main_res, (apk, bpk, c_d, m, n, k, wall_ms) = run_workload(a.workload, a.steps, a.warmup)
     line = {
