@@ -54,7 +54,11 @@ int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, int k, void 
  * made by LAUNCH_KERNEL_IF_CONDITION / IGemmConfig (kernel.cu:321-332, 23-50)
  * from the constexpr table in configs.cu:19-689; used by the autotuner that
  * regenerates this library's per-shape table.  cfg = QM_CFG_AUTO behaves as
- * qm_gemm_i4.
+ * qm_gemm_i4.  Otherwise: configuration id in bits 0..15, tile raster group
+ * height in bits 16..23 (0 = default), K split in bits 24..29 (0 or 1 = none;
+ * above 1 only for the pipelined "q" configurations: C is zero-filled by a first
+ * kernel and the partial sums are added into it with integer atomics, still
+ * exact, still one enqueue on the caller's stream).
  */
 int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg);
 

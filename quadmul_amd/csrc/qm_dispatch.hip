@@ -162,9 +162,9 @@ static const ConfigDesc g_configs[] = {
 #define QM_TILE(tu, BM, BN, BK, WGM, WGN, MODE)                                                        \
     {"t" QM_STR(BM) "x" QM_STR(BN) "x" QM_STR(BK) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_m" QM_STR(MODE), \
      KIND_TILE, BM, BN, BK, (WGM) * (WGN), MODE, &QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)},
-#define QM_TILE16(tu, BM, BN, WGM, WGN)                                                              \
-    {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN), KIND_TILE16, BM, BN, 128, (WGM) * (WGN), 0, \
-     &QM_TILE16_FN(BM, BN, WGM, WGN)},
+#define QM_TILE16(tu, BM, BN, WGM, WGN, ST, OCC)                                                              \
+    {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_s" QM_STR(ST) "o" QM_STR(OCC), KIND_TILE16, BM, BN, 128, \
+     (WGM) * (WGN), 0, &QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)},
 #define QM_SKINNY(FM, FN, NW, U)                                                     \
     {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
      &QM_SKINNY_FN(FM, FN, NW, U)},
@@ -206,45 +206,53 @@ static bool config_supports(int cfg, int m, int n, int k, int ptr_align)
 struct TableEntry {
     int m, n, k;
     const char *config;
-    int group_m;
+    int group_m, ksplit;
 };
 static const TableEntry g_table[] = {
 #include "qm_tile_table.inc"
-    {0, 0, 0, nullptr, 0},
+    {0, 0, 0, nullptr, 0, 0},
 };
 
 struct Choice {
-    int cfg, group_m;
+    int cfg, group_m, ksplit;
 };
 
 static Choice heuristic(int m, int n, int k, int ptr_align)
 {
-    if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1};
+    if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
     if (m <= 64) {
         const int fm = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
         const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w8_u2");
         const int id = find_config(name);
-        if (id >= 0) return {id, 1};
+        if (id >= 0) return {id, 1, 1};
     }
     // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency),
     // over the configurations that can run this K.  Efficiencies are measured ratios.
     static const struct { const char *name; double eff; } cands[] = {
-        {"q256x256_w2x2", 1.00}, {"q256x128_w2x2", 0.82}, {"q128x256_w2x2", 0.82}, {"q128x128_w2x2", 0.66},
+        {"q256x256_w2x2_s4o1", 1.00}, {"q256x128_w2x2_s4o1", 0.82}, {"q128x256_w2x2_s4o1", 0.82}, {"q128x128_w2x2_s4o1", 0.66},
         {"t256x256x128_w4x2_m0", 0.78}, {"t128x128x128_w2x2_m0", 0.60}, {"t64x128x128_w2x2_m0", 0.40},
         {"t128x64x128_w2x2_m0", 0.40},  {"t64x64x128_w2x2_m0", 0.30},
     };
-    int best = 0;
+    int best = 0, best_ks = 1;
     double best_cost = 1e300;
     for (const auto &c : cands) {
         const int id = find_config(c.name);
         if (id < 0 || !config_supports(id, m, n, k, ptr_align)) continue;
         const ConfigDesc &d = g_configs[id];
         const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
-        const long long rounds = (tiles + 255) / 256;
-        const double cost = (double)rounds * d.bm * d.bn / c.eff;
-        if (cost < best_cost) { best_cost = cost; best = id; }
+        // Few tiles and a very long K: the pipelined kernel can split K over several
+        // workgroups per tile.  The partial sums meet in C through 4-byte atomics, which
+        // are slow enough that this only pays when each split keeps a long K of its own
+        // (measured: wins at K = 28672, loses at K = 8192).
+        int ks = 1;
+        if (d.kind == KIND_TILE16)
+            while (ks < 4 && tiles * ks * 2 <= 256 && (k / 128) / (ks * 2) >= 48) ks *= 2;
+        const long long rounds = (tiles * ks + 255) / 256;
+        const double cost = (double)rounds * d.bm * d.bn / c.eff / ks * (ks > 1 ? 1.25 : 1.0);
+        if (cost < best_cost) { best_cost = cost; best = id; best_ks = ks; }
     }
-    return {best, 4};
+    const int ksplit = best_ks;
+    return {best, 4, ksplit};
 }
 
 static Choice select_config(int m, int n, int k, int ptr_align)
@@ -257,7 +265,7 @@ static Choice select_config(int m, int n, int k, int ptr_align)
     for (size_t i = 0; g_table[i].config; ++i)
         if (g_table[i].m == m && g_table[i].n == n && g_table[i].k == k && resolved[i] >= 0 &&
             config_supports(resolved[i], m, n, k, ptr_align))
-            return {resolved[i], g_table[i].group_m};
+            return {resolved[i], g_table[i].group_m, g_table[i].ksplit > 0 ? g_table[i].ksplit : 1};
     return heuristic(m, n, k, ptr_align);
 }
 
@@ -310,11 +318,21 @@ QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n
     } else {
         ch.cfg = cfg & 0xFFFF;
         ch.group_m = (cfg >> 16) & 0xFF;
+        ch.ksplit = (cfg >> 24) & 0x3F;
         if (ch.group_m == 0) ch.group_m = 4;
+        if (ch.ksplit == 0) ch.ksplit = 1;
         if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
+        if (ch.ksplit > 1 && g_configs[ch.cfg].kind != KIND_TILE16) return QM_ERR_CONFIG;
     }
     const GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(C), m, n, k};
-    const hipError_t e = g_configs[ch.cfg].launch(p, s, ch.group_m);
+    if (ch.ksplit > 1) {
+        // split-K partial sums meet in C by integer atomic adds: C starts from zero
+        const size_t cnt = (size_t)m * (size_t)n;
+        fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(C), cnt);
+        const hipError_t ez = hipGetLastError();
+        if (ez != hipSuccess) return fail_launch(ez);
+    }
+    const hipError_t e = g_configs[ch.cfg].launch(p, s, ch.group_m | (ch.ksplit << 8));
     return e == hipSuccess ? QM_OK : fail_launch(e);
 }
 
@@ -327,7 +345,7 @@ QM_EXPORT int qm_select_config(int m, int n, int k, int ptr_align)
 {
     if (m < 1 || n < 1 || k < 2 || (k & 1)) return QM_ERR_SHAPE;
     const Choice ch = select_config(m, n, k, ptr_align);
-    return ch.cfg | (ch.group_m << 16);
+    return ch.cfg | (ch.group_m << 16) | (ch.ksplit << 24);
 }
 
 QM_EXPORT int qm_num_configs(void) { return g_num_configs; }

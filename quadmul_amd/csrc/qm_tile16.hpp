@@ -48,8 +48,15 @@ __device__ __forceinline__ void mfma16_acc(v4i &acc, const v4i &s0, const v4i &s
     asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(s0), "v"(s1));
 }
 
-template <int BM_, int BN_, int WGM_, int WGN_>
+// Wait states between the last MFMA into `acc` and its first ordinary reader.
+__device__ __forceinline__ void mfma16_settle(v4i &acc)
+{
+    asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc));
+}
+
+template <int BM_, int BN_, int WGM_, int WGN_, int STAGES_ = 4, int OCC_ = 1>
 struct Tile16Cfg {
+    static constexpr int OCC = OCC_;  // workgroups meant to share a CU (sets the register budget)
     static constexpr int BM = BM_, BN = BN_, BK = 128, WGM = WGM_, WGN = WGN_;
     static constexpr int WAVES = WGM * WGN, THREADS = 64 * WAVES;
     static constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -57,20 +64,22 @@ struct Tile16Cfg {
     static constexpr int PITCH = 64;                  // packed bytes per row per K-step
     static constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int STAGES = 4;
+    static constexpr int STAGES = STAGES_;  // LDS ring depth: 4, or 5 for one more K-step of DMA latency cover
     static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
     // one DMA piece = one wave-wide 16-byte-per-lane load = 16 rows x 64 bytes
     static constexpr int A_PIECES = BM / 16 / WAVES, B_PIECES = BN / 16 / WAVES;
     static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile is a multiple of 16x16");
     static_assert(BM % (16 * WAVES) == 0 && BN % (16 * WAVES) == 0, "DMA pieces must divide evenly among the waves");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
+    static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
+    static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
     static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
     static_assert((12 * FN) % FM == 0, "B widening must split evenly over the sub-steps");
 };
 
 template <class Cfg>
-__global__ void __launch_bounds__(Cfg::THREADS)
-gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const int group_m)
+__global__ void __launch_bounds__(Cfg::THREADS, Cfg::OCC * Cfg::THREADS / 256)
+gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const int group_m, const int ksplit)
 {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, FM = Cfg::FM, FN = Cfg::FN;
     constexpr int PITCH = Cfg::PITCH, STAGE = Cfg::STAGE_BYTES, WAVES = Cfg::WAVES;
@@ -83,15 +92,28 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     const int wm = wave / Cfg::WGN, wn = wave % Cfg::WGN;
     const int r = lane & 15, g = lane >> 4;
 
-    const int pid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    // workgroup -> (K split, tile): XCD-contiguous id, tiles in columns of group_m
+    const int gid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int ntiles = tiles_m * tiles_n;
+    // (readfirstlane: the quotient is computed on the vector ALU; everything derived from it
+    // is wave-uniform and belongs in scalar registers)
+    const int ks = __builtin_amdgcn_readfirstlane(gid / ntiles), pid = gid - ks * ntiles;
     const int width = group_m * tiles_n;
     const int first_m = (pid / width) * group_m;
     const int gsz = min(tiles_m - first_m, group_m);
-    const int m0 = (first_m + (pid % width) % gsz) * BM;
-    const int n0 = ((pid % width) / gsz) * BN;
+    const int m0 = __builtin_amdgcn_readfirstlane((first_m + (pid % width) % gsz) * BM);
+    const int n0 = __builtin_amdgcn_readfirstlane(((pid % width) / gsz) * BN);
 
+    // This workgroup contracts K-steps [kt0, kt0 + KT) of the K / 128 in total (all of
+    // them unless the launch splits K; then the partial sums meet in C by atomic adds
+    // and the host has zero-filled C beforehand).
     const int Kb = p.K >> 1;
-    const int KT = p.K / BK;  // K is a multiple of 128 for this kernel
+    const int kt_all = p.K / BK;  // K is a multiple of 128 for this kernel
+    const int kps = (kt_all + ksplit - 1) / ksplit;
+    const int kt0 = __builtin_amdgcn_readfirstlane(min(ks * kps, kt_all - 1));
+    const int KT = __builtin_amdgcn_readfirstlane(min(kps, kt_all - ks * kps));  // >= 1: the launcher never creates an empty split
+    // (no early exit here: a branch around the whole body costs the register allocator
+    // dearly; an empty split would simply run no K-step and add zeros)
 
     // ---- global -> LDS: piece q of this wave covers tile rows (q*WAVES + wave)*16 .. +15.
     // The hardware puts lane l's 16 bytes at (wave-uniform LDS base) + 16*l, i.e. row l/4,
@@ -113,7 +135,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // piece index -> (operand, piece): issues one wave-wide load of tile `kt` into `stage_byte`.
     // Tiles past the end re-read the last tile; they land in a stage nobody reads any more.
     auto dma_piece = [&](int piece, int stage_byte, int kt) {
-        const int kofs = min(kt, KT - 1) * (BK / 2);
+        const int kofs = (kt0 + max(min(kt, KT - 1), 0)) * (BK / 2);
         if (piece < A_PIECES) {
             const uint32_t dst = dma_lds + stage_byte + piece * WAVES * 16 * PITCH;
             const uint8_t *src = p.A + kofs;
@@ -146,12 +168,13 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    // ---- prologue: tiles 0, 1, 2 on their way into stages 0, 1, 2; wait for 0 and 1 ----
+    // ---- prologue: tiles 0 .. STAGES-2 on their way into stages 0 .. STAGES-2; wait for 0 and 1 ----
+    constexpr int STAGES = Cfg::STAGES, AHEAD = STAGES - 1;  // tile kt+AHEAD is issued during K-step kt
 #pragma unroll
-    for (int t = 0; t < 3; ++t)
+    for (int t = 0; t < AHEAD; ++t)
 #pragma unroll
         for (int q = 0; q < NP; ++q) dma_piece(q, t * STAGE, t);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NP) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 2) * NP) : "memory");
     __syncthreads();
 
     // B fragments of the current tile (widened) and of the next (being widened); the two
@@ -164,7 +187,10 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     x16_expand(read_a(0, 0), a_ev[0], a_od[0]);
     a_pk[1] = read_a(0, 1);
 
-    int cur = 0, nxt = STAGE, lnd = 2 * STAGE, fly = 3 * STAGE;  // byte offsets of the ring stages
+    // byte offsets of the ring stages: tile kt, kt+1, ..., and the one being (re)filled
+    int ring[STAGES];
+#pragma unroll
+    for (int t = 0; t < STAGES; ++t) ring[t] = t * STAGE;
 
     // Widening op k (0..11) of a packed fragment: dword k/3; part 0: shift, 1: mask -> even
     // nibbles, 2: mask -> odd nibbles.
@@ -175,6 +201,11 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         else od[d] = (int)((uint32_t)pk[d] & mask);
     };
 
+    // The nibble mask lives in an SGPR (opaque to the compiler): a VALU instruction with
+    // an SGPR operand is half the size of one with a 32-bit literal.
+    uint32_t amask;
+    asm volatile("s_mov_b32 %0, 0xf0f0f0f0" : "=s"(amask));
+
     auto k_step = [&](const int kt, auto bs_tag) {
         constexpr int bs = decltype(bs_tag)::value;  // B register set holding tile kt
         constexpr int SLOTS = 2 * FN;                // MFMAs per sub-step
@@ -182,7 +213,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         constexpr int NOPS = 12 + BSHARE;            // VALU ops per sub-step, spread over slots 1..SLOTS-1
         // The loop runs K-steps in pairs; when the number of tiles is odd the last step
         // contracts a tile that does not exist, so its B operand is widened to zero.
-        const uint32_t bmask = kt + 1 < KT ? 0xF0F0F0F0u : 0u;
+        const uint32_t bmask = kt + 1 < KT ? amask : 0u;
         static_for<0, FM>([&](auto i_) {
             constexpr int i = decltype(i_)::value;
             constexpr int pa = i & 1;
@@ -196,10 +227,10 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     //    sub-step, and the A fragment two sub-steps ahead --
                     static_for<0, FN>([&](auto j_) {
                         constexpr int j = decltype(j_)::value;
-                        if constexpr ((12 * j) / BSHARE == i) b_pk[j & 1] = read_b(nxt, j);
+                        if constexpr ((12 * j) / BSHARE == i) b_pk[j & 1] = read_b(ring[1], j);
                     });
                     constexpr int i2 = i + 2;
-                    a_pk[pa] = read_a(i2 >= FM ? nxt : cur, i2 % FM);
+                    a_pk[pa] = read_a(i2 >= FM ? ring[1] : ring[0], i2 % FM);
                 } else {
                     // -- this slot's share of the widening work: ops [lo, hi) of the sub-step's
                     //    list: 12 ops for the next A fragment, then BSHARE ops of B(kt+1) --
@@ -207,7 +238,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     static_for<lo, hi>([&](auto o_) {
                         constexpr int o = decltype(o_)::value;
                         if constexpr (o < 12) {
-                            widen_op(std::integral_constant<int, o>{}, a_pk[pa ^ 1], a_ev[pa ^ 1], a_od[pa ^ 1], 0xF0F0F0F0u);
+                            widen_op(std::integral_constant<int, o>{}, a_pk[pa ^ 1], a_ev[pa ^ 1], a_od[pa ^ 1], amask);
                         } else {
                             constexpr int gop = i * BSHARE + (o - 12);  // index into the K-step's B op list
                             constexpr int j = gop / 12;
@@ -219,29 +250,32 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 if constexpr (s == SLOTS - 1) {
                     static_for<0, NP>([&](auto q_) {
                         constexpr int q = decltype(q_)::value;
-                        if constexpr (q * FM / NP == i) dma_piece(q, fly, kt + 3);
+                        if constexpr (q * FM / NP == i) dma_piece(q, ring[STAGES - 1], kt + AHEAD);
                     });
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
-        // Tile kt+2 (issued one K-step ago) must have landed, and every wave must be done
-        // reading stage `cur`, before the roles rotate; tile kt+3 stays in flight.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NP) : "memory");
-        const int t = cur;
-        cur = nxt;
-        nxt = lnd;
-        lnd = fly;
-        fly = t;
+        // Tile kt+2 must have landed, and every wave must be done reading tile kt's stage,
+        // before the roles rotate; the younger tiles stay in flight.
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((AHEAD - 2) * NP) : "memory");
+        const int t = ring[0];
+#pragma unroll
+        for (int u = 0; u + 1 < STAGES; ++u) ring[u] = ring[u + 1];
+        ring[STAGES - 1] = t;
     };
 
     for (int kt = 0; kt < KT; kt += 2) {
         k_step(kt, std::integral_constant<int, 0>{});
         k_step(kt + 1, std::integral_constant<int, 1>{});
     }
-    // drain the DMA before the LDS is released; let the last MFMAs retire before their
-    // accumulators are read (the compiler does not know the asm statements were MFMAs)
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    // Drain the DMA before the LDS is released, and let the last MFMAs retire before their
+    // accumulators are read: the compiler does not know the asm statements were MFMAs, so
+    // the wait is tied to the accumulators written last (it cannot be scheduled around).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    static_for<(FN > 4 ? FN - 4 : 0), FN>([&](auto j_) {
+        mfma16_settle(acc[FM - 1][decltype(j_)::value]);
+    });
 
     // ---- epilogue: drop the factor 256, guarded 16-byte stores ----
     const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
@@ -255,7 +289,13 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             const int n = n0 + wn * Cfg::WN + j * 16 + g * 4;
             v4i v = acc[i][j];
             v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
-            if (vec_ok && n + 3 < p.N) {
+            if (ksplit > 1) {
+                // every partial accumulator is a multiple of 256, so the shifted partials add
+                // up to the shifted total; integer atomics make the order irrelevant
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else if (vec_ok && n + 3 < p.N) {
                 *reinterpret_cast<v4i *>(crow + n) = v;
             } else {
                 if (n < p.N) crow[n] = v.x;

@@ -10,16 +10,39 @@
 
 namespace qm {
 
+// opt: tile raster group height in bits 0..7, K split in bits 8..15 (pipelined kernel only;
+// the caller has zero-filled C when the split is above 1)
 template <class Cfg, class Kernel>
-static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t stream, int group_m)
+static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
 {
     static bool lds_ok[QM_MAX_DEVICES] = {};
     hipError_t e = ensure_dynamic_lds(kernel, Cfg::LDS_BYTES, lds_ok);
     if (e != hipSuccess) return e;
     const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
+    int group_m = opt & 0xFF;
     if (group_m < 1) group_m = 1;
     if (group_m > tiles_m) group_m = tiles_m;
     kernel<<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, tiles_m, tiles_n, group_m);
+    return hipGetLastError();
+}
+
+template <class Cfg, class Kernel>
+static hipError_t launch_tiled_splitk(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
+{
+    static bool lds_ok[QM_MAX_DEVICES] = {};
+    hipError_t e = ensure_dynamic_lds(kernel, Cfg::LDS_BYTES, lds_ok);
+    if (e != hipSuccess) return e;
+    const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
+    int group_m = opt & 0xFF, ksplit = (opt >> 8) & 0xFF;
+    if (group_m < 1) group_m = 1;
+    if (group_m > tiles_m) group_m = tiles_m;
+    if (ksplit < 1) ksplit = 1;
+    {
+        // no empty splits: with kps K-steps per split, only ceil(kt / kps) splits have work
+        const int kt = p.K / Cfg::BK, kps = (kt + ksplit - 1) / ksplit;
+        ksplit = (kt + kps - 1) / kps;
+    }
+    kernel<<<dim3(tiles_m * tiles_n * ksplit), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, tiles_m, tiles_n, group_m, ksplit);
     return hipGetLastError();
 }
 
@@ -33,12 +56,12 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
         return launch_tiled<Cfg>(&gemm_tile_kernel<Cfg>, p, s, gm);                             \
     }                                                                                           \
     }
-#define QM_TILE16_DEF(BM, BN, WGM, WGN)                                                 \
-    namespace qm {                                                                      \
-    hipError_t QM_TILE16_FN(BM, BN, WGM, WGN)(const GemmArgs &p, hipStream_t s, int gm) \
-    {                                                                                   \
-        using Cfg = Tile16Cfg<BM, BN, WGM, WGN>;                                        \
-        return launch_tiled<Cfg>(&gemm_tile16_kernel<Cfg>, p, s, gm);                   \
+#define QM_TILE16_DEF(BM, BN, WGM, WGN, ST, OCC)                                                 \
+    namespace qm {                                                                               \
+    hipError_t QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &p, hipStream_t s, int gm) \
+    {                                                                                            \
+        using Cfg = Tile16Cfg<BM, BN, WGM, WGN, ST, OCC>;                                        \
+        return launch_tiled_splitk<Cfg>(&gemm_tile16_kernel<Cfg>, p, s, gm);                   \
     }                                                                                   \
     }
 
@@ -52,10 +75,6 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 #define QM_PICK_5(...)
 #define QM_PICK_6(...)
 #define QM_PICK_7(...)
-#define QM_PICK_8(...)
-#define QM_PICK_9(...)
-#define QM_PICK_10(...)
-#define QM_PICK_11(...)
 #define QM_PICK16_0(...)
 #define QM_PICK16_1(...)
 #define QM_PICK16_2(...)
@@ -64,10 +83,6 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 #define QM_PICK16_5(...)
 #define QM_PICK16_6(...)
 #define QM_PICK16_7(...)
-#define QM_PICK16_8(...)
-#define QM_PICK16_9(...)
-#define QM_PICK16_10(...)
-#define QM_PICK16_11(...)
 #if QM_TU == 0
 #undef QM_PICK_0
 #define QM_PICK_0(...) QM_TILE_DEF(__VA_ARGS__)
@@ -108,26 +123,6 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 #define QM_PICK_7(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_7
 #define QM_PICK16_7(...) QM_TILE16_DEF(__VA_ARGS__)
-#elif QM_TU == 8
-#undef QM_PICK_8
-#define QM_PICK_8(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_8
-#define QM_PICK16_8(...) QM_TILE16_DEF(__VA_ARGS__)
-#elif QM_TU == 9
-#undef QM_PICK_9
-#define QM_PICK_9(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_9
-#define QM_PICK16_9(...) QM_TILE16_DEF(__VA_ARGS__)
-#elif QM_TU == 10
-#undef QM_PICK_10
-#define QM_PICK_10(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_10
-#define QM_PICK16_10(...) QM_TILE16_DEF(__VA_ARGS__)
-#elif QM_TU == 11
-#undef QM_PICK_11
-#define QM_PICK_11(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_11
-#define QM_PICK16_11(...) QM_TILE16_DEF(__VA_ARGS__)
 #else
 #error "QM_TU out of range"
 #endif

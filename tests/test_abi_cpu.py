@@ -48,7 +48,7 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4(None, None, None, 4, 0, 4, None) == 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 4, 4, 4, None, 9999) == -3
     assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("t128x128x128_w2x2_m0")) == -3
-    assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 160, None, qm.config_id("q256x256_w2x2")) == -3
+    assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 160, None, qm.config_id("q256x256_w2x2_s4o1")) == -3
     assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
     assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
     assert lib.qm_unpack_i4(None, one, 4, 8, None) == -1
@@ -75,6 +75,10 @@ def test_selection_rules():
     assert name(4096, 4096, 4096 + 32).startswith("t")  # K % 32 == 0 only: plain tile kernel
     for m in (1, 16, 64):
         assert name(m, 4096, 4096).startswith("s"), m
+    # few tiles, long K: the pipelined kernel with K split over several workgroups per tile
+    code = qm.select_config(128, 8192, 28672)
+    assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
+    assert (qm.select_config(8192, 8192, 8192) >> 24) & 0x3F == 1
     assert name(100, 100, 30) == "generic"          # K % 32 != 0: no 16-byte chunks
     assert name(128, 128, 4096, 4) == "generic"     # operands not 16-byte aligned
     assert name(128, 128, 262144) == "generic"      # beyond the exact range of the x16 widening

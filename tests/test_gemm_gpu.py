@@ -46,10 +46,13 @@ def test_every_config_matches_oracle(oracle_mod, shape):
     for cfg, name in enumerate(qm.config_names()):
         if not qm.config_supports(cfg, m, n, k):
             continue
-        for gm in (1, 3):
-            got = run_gemm(ap, bp, m, n, k, cfg | (gm << 16))
+        # raster group heights; K splits (pipelined kernel only: 3 does not divide the K-steps,
+        # 8 leaves some splits empty on short K)
+        variants = [(1, 1), (3, 1)] + ([(2, 2), (1, 3), (4, 8)] if name.startswith("q") else [])
+        for gm, ks in variants:
+            got = run_gemm(ap, bp, m, n, k, cfg | (gm << 16) | (ks << 24))
             bad = oracle_mod.compare(got, want)
-            assert bad == -1, f"{name} group_m={gm}: first mismatch at flat index {bad}: got {got.flat[bad]} want {want.flat[bad]}"
+            assert bad == -1, f"{name} group_m={gm} ksplit={ks}: first mismatch at flat index {bad}: got {got.flat[bad]} want {want.flat[bad]}"
         ran += 1
     assert ran >= 2
     got = run_gemm(ap, bp, m, n, k)
@@ -118,6 +121,8 @@ def test_extremes_closed_form_on_every_config(shape):
             continue
         assert (run_gemm(lo_a, lo_b, m, n, k, cfg) == 64 * k).all(), name   # largest positive accumulator
         assert (run_gemm(lo_a, hi_b, m, n, k, cfg) == -56 * k).all(), name  # most negative accumulator
+        if name.startswith("q"):  # split K: partial sums meet by atomic adds
+            assert (run_gemm(lo_a, hi_b, m, n, k, cfg | (4 << 24)) == -56 * k).all(), name
 
 
 def test_largest_exact_k_and_beyond(oracle_mod):
