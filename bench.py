@@ -196,7 +196,7 @@ def main(argv=None):
     a = ap.parse_args(argv)
     if a.gpus != 1:
         print("bench.py: this hot path is a single-GPU kernel and every box here has one GPU; "
-              "run with --gpus 1 (sharding over M or N needs no exchange and is described in DESIGN.md)", file=sys.stderr)
+              "run with --gpus 1 (row blocks of A or of B shard with no exchange; a split of K needs one int32 all-reduce)", file=sys.stderr)
         return 2
     import torch
 

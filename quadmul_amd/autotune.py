@@ -6,7 +6,7 @@ times every compiled-in configuration that supports a shape, over a few raster
 group heights, on the GPU it runs on, checks each candidate bit-exactly against
 the library's own generic kernel, and writes the winners as table rows.
 
-    python -m quadmul_amd.autotune --shapes baseline --json out.json --emit table.inc
+    python -m quadmul_amd.autotune --shapes named --json out.json --emit table.inc
 
 Timing: HIP events on the stream the kernels are launched on, back-to-back
 launches for at least ``--min-ms`` per sample, median of ``--reps`` samples.
@@ -24,7 +24,7 @@ import torch
 
 import quadmul_amd as qm
 
-BASELINE_SHAPES: List[Tuple[int, int, int]] = [
+NAMED_SHAPES: List[Tuple[int, int, int]] = [
     (1024, 1024, 1024), (4096, 4096, 4096),
     (1, 4096, 4096), (16, 4096, 4096), (64, 4096, 4096),
     (2048, 11008, 4096), (2048, 4096, 11008), (2048, 12288, 4096),
@@ -155,12 +155,12 @@ def emit_table(tuned: List[Dict], path: str) -> None:
 
 
 def parse_shapes(spec: str) -> List[Tuple[int, int, int]]:
-    if spec == "baseline":
-        return BASELINE_SHAPES
+    if spec in ("named", "baseline"):
+        return NAMED_SHAPES
     if spec == "reference":
         return REFERENCE_SHAPES
     if spec == "all":
-        return BASELINE_SHAPES + REFERENCE_SHAPES
+        return NAMED_SHAPES + REFERENCE_SHAPES
     out = []
     for part in spec.split(","):
         m, n, k = (int(x) for x in part.lower().split("x"))
@@ -170,7 +170,7 @@ def parse_shapes(spec: str) -> List[Tuple[int, int, int]]:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("--shapes", default="baseline", help="baseline | reference | all | MxNxK[,MxNxK...]")
+    ap.add_argument("--shapes", default="named", help="named | reference | all | MxNxK[,MxNxK...]")
     ap.add_argument("--group-m", default="1,2,4,8,16", help="raster group heights to try for tile kernels")
     ap.add_argument("--min-ms", type=float, default=20.0)
     ap.add_argument("--reps", type=int, default=3)

@@ -8,6 +8,7 @@
 // The argument checks the reference left commented out (extension.cpp:11-15) are
 // live here; a non-zero status from the library is raised as RuntimeError.
 #include <torch/extension.h>
+#include <torch/library.h>
 
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
@@ -80,7 +81,18 @@ torch::Tensor unpack(torch::Tensor packed)
     return out;
 }
 
+// Dispatcher-visible form of the same op (schema + mutation annotation), so that callers
+// under torch.compile / export can keep `torch.ops.quadmul.gemm(a, b, c, m, n, k)` in the
+// graph.  The reference has only the pybind function (extension.cpp:26-29), which a tracer
+// cannot see through.  c is written in place; nothing is returned.
+void gemm_meta(const torch::Tensor &, const torch::Tensor &, torch::Tensor &, int64_t, int64_t, int64_t) {}
+void gemm_op(const torch::Tensor &a, const torch::Tensor &b, torch::Tensor &c, int64_t m, int64_t n, int64_t k) { gemm(a, b, c, m, n, k); }
+
 }  // namespace
+
+TORCH_LIBRARY(quadmul, m) { m.def("gemm(Tensor a, Tensor b, Tensor(c!) c, int m, int n, int k) -> ()"); }
+TORCH_LIBRARY_IMPL(quadmul, CUDA, m) { m.impl("gemm", &gemm_op); }
+TORCH_LIBRARY_IMPL(quadmul, Meta, m) { m.impl("gemm", &gemm_meta); }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {

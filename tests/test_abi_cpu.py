@@ -36,6 +36,24 @@ def test_extension_module_imports_and_mirrors_reference_entry_point():
     assert quadmul.num_configs() == qm.num_configs()
 
 
+def test_dispatcher_op_is_registered_with_a_mutation_schema():
+    import torch
+    import quadmul  # noqa: F401  (registers torch.ops.quadmul.gemm)
+
+    schema = torch.ops.quadmul.gemm.default._schema
+    assert [a.name for a in schema.arguments] == ["a", "b", "c", "m", "n", "k"]
+    assert schema.arguments[2].alias_info is not None and schema.arguments[2].alias_info.is_write
+    assert len(schema.returns) == 0
+    # the Meta kernel lets a tracer run the op without data
+    a = torch.empty((4, 16), dtype=torch.int8, device="meta")
+    c = torch.empty((4, 4), dtype=torch.int32, device="meta")
+    assert torch.ops.quadmul.gemm(a, a, c, 4, 4, 32) is None
+    # no CPU kernel: the product path is the GPU one only
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.quadmul.gemm(torch.zeros((4, 16), dtype=torch.int8), torch.zeros((4, 16), dtype=torch.int8),
+                               torch.zeros((4, 4), dtype=torch.int32), 4, 4, 32)
+
+
 def test_status_codes_without_a_gpu():
     lib = qm.library()
     one = ctypes.c_void_p(4096)  # never dereferenced: the checks come first

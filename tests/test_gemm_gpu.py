@@ -194,6 +194,30 @@ def test_extension_module_runs_on_side_stream_and_under_graph_replay(oracle_mod)
         assert oracle_mod.compare(c3.cpu().numpy(), want) == -1
 
 
+def test_dispatcher_op_eager_and_traced(oracle_mod):
+    import quadmul  # noqa: F401
+
+    m, n, k = 130, 200, 640
+    a, b = make_operands(m, n, k, SEED_BASE + 3200)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    c_d = poisoned_c(m, n, DEV)
+    torch.ops.quadmul.gemm(a_d, b_d, c_d, m, n, k)
+    torch.cuda.synchronize()
+    assert oracle_mod.compare(c_d.cpu().numpy(), want) == -1
+
+    def fn(x, y):
+        out = torch.full((m, n), 0x7F7F7F7F, dtype=torch.int32, device=x.device)
+        torch.ops.quadmul.gemm(x, y, out, m, n, k)
+        return out
+
+    traced = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    got = traced(a_d, b_d)
+    torch.cuda.synchronize()
+    assert oracle_mod.compare(got.cpu().numpy(), want) == -1
+
+
 def test_pack_unpack_kernels(oracle_mod):
     from util import make_values
 
@@ -211,14 +235,14 @@ def test_pack_unpack_kernels(oracle_mod):
 
 
 # ------------------------------------------------------------------ the named workloads
-BASELINE_SHAPES = [
+NAMED_SHAPES = [
     (0, 1024, 1024, 1024), (1, 4096, 4096, 4096),
     (2, 1, 4096, 4096), (3, 16, 4096, 4096), (4, 64, 4096, 4096),
     (5, 2048, 11008, 4096), (6, 2048, 4096, 11008), (7, 2048, 12288, 4096),
 ]
 
 
-@pytest.mark.parametrize("row", BASELINE_SHAPES, ids=lambda r: "x".join(map(str, r[1:])))
+@pytest.mark.parametrize("row", NAMED_SHAPES, ids=lambda r: "x".join(map(str, r[1:])))
 def test_baseline_configs_full_compare(oracle_mod, row):
     i, m, n, k = row
     a, b = make_operands(m, n, k, SEED_BASE + i)
