@@ -58,7 +58,9 @@ int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, int k, void 
  * height in bits 16..23 (0 = default), K split in bits 24..29 (0 or 1 = none;
  * above 1 only for the pipelined "q" configurations: C is zero-filled by a first
  * kernel and the partial sums are added into it with integer atomics, still
- * exact, still one enqueue on the caller's stream).
+ * exact, still one enqueue on the caller's stream).  Bit 30, "q" configurations
+ * only: launch one workgroup per (K split, tile) instead of the default persistent
+ * grid whose workgroups each run several tiles back to back.
  */
 int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg);
 

@@ -116,26 +116,32 @@ def tune_shape(m: int, n: int, k: int, device, group_ms: Iterable[int], min_ms: 
         gms = list(group_ms) if name[0] in "tq" else [1]
         # K split (pipelined kernel only): worth trying when the tiles alone cannot fill the GPU
         kss = [1]
+        tiles = 0
         if name[0] == "q":
             bm, bn = (int(x) for x in name[1:].split("_")[0].split("x"))
             tiles = -(-m // bm) * -(-n // bn)
             kss = [ks for ks in (1, 2, 4, 8) if ks == 1 or (tiles * ks <= 512 and (k // 128) // ks >= 4)]
-        for gm, ks in [(g_, k_) for k_ in kss for g_ in (gms if k_ == 1 else gms[:1])]:
-            code = cfg | (gm << 16) | (ks << 24)
+        # (K split, group height, one-item-per-workgroup flag); the flag only changes the launch
+        # when there are more work items than the device holds workgroups of the pipelined kernel
+        variants = [(g_, k_, 0) for k_ in kss for g_ in (gms if k_ == 1 else gms[:1])]
+        if name[0] == "q" and tiles > 256:
+            variants += [(g_, 1, 1) for g_ in gms]
+        for gm, ks, spread in variants:
+            code = cfg | (gm << 16) | (ks << 24) | (spread << 30)
             c.fill_(0x7F7F7F7F)
             qm.gemm_cfg(a, b, c, m, n, k, code)
             if ref is None:
                 ref = c.clone()
             if not torch.equal(c, ref):
-                raise RuntimeError(f"{name} group_m={gm} ksplit={ks} disagrees with the cross-check result on {m}x{n}x{k}")
+                raise RuntimeError(f"{name} group_m={gm} ksplit={ks} spread={spread} disagrees with the cross-check result on {m}x{n}x{k}")
             ms = time_launches(lambda: qm.gemm_cfg(a, b, c, m, n, k, code), min_ms, reps)
-            results.append({"config": name, "group_m": gm, "ksplit": ks, "ms": ms, "tops": ops / ms / 1e9,
+            results.append({"config": name, "group_m": gm, "ksplit": ks, "spread": spread, "ms": ms, "tops": ops / ms / 1e9,
                             "gbs": algorithmic_bytes(m, n, k) / ms / 1e6})
             if verbose:
-                print(f"  {m}x{n}x{k} {name:28s} gm={gm:2d} ks={ks} {ms*1e3:9.1f} us {ops/ms/1e9:8.1f} TOPS", flush=True)
+                print(f"  {m}x{n}x{k} {name:28s} gm={gm:2d} ks={ks} spread={spread} {ms*1e3:9.1f} us {ops/ms/1e9:8.1f} TOPS", flush=True)
     results.sort(key=lambda r: r["ms"])
     best = results[0]
-    print(f"{m}x{n}x{k}: best {best['config']} gm={best['group_m']} ks={best['ksplit']} {best['ms']*1e3:.1f} us "
+    print(f"{m}x{n}x{k}: best {best['config']} gm={best['group_m']} ks={best['ksplit']} spread={best['spread']} {best['ms']*1e3:.1f} us "
           f"{best['tops']:.1f} TOPS ({100*best['tops']/INT8_PEAK_TOPS:.1f}% int8 peak) "
           f"{best['gbs']:.0f} GB/s ({100*best['gbs']/HBM_PEAK_GBS:.1f}% HBM)", flush=True)
     return {"m": m, "n": n, "k": k, "best": best, "all": results}
@@ -143,7 +149,8 @@ def tune_shape(m: int, n: int, k: int, device, group_ms: Iterable[int], min_ms: 
 
 def emit_table(tuned: List[Dict], path: str) -> None:
     lines = [
-        "// Per-shape kernel choice measured on MI355X: {M, N, K, \"config name\", group_m, ksplit}.",
+        "// Per-shape kernel choice measured on MI355X: {M, N, K, \"config name\", group_m, ksplit,",
+        "// one item per workgroup}.",
         "// Written by quadmul_amd/autotune.py; shapes not listed use the cost model in",
         "// qm_dispatch.hip.  Counterpart of the reference's A40 table (configs.cu:19-689).",
     ]

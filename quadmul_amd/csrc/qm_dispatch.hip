@@ -207,6 +207,7 @@ struct TableEntry {
     int m, n, k;
     const char *config;
     int group_m, ksplit;
+    int spread;  // 1: one work item per workgroup instead of a persistent grid (pipelined kernel)
 };
 static const TableEntry g_table[] = {
 #include "qm_tile_table.inc"
@@ -215,6 +216,7 @@ static const TableEntry g_table[] = {
 
 struct Choice {
     int cfg, group_m, ksplit;
+    int spread = 0;
 };
 
 static Choice heuristic(int m, int n, int k, int ptr_align)
@@ -265,7 +267,7 @@ static Choice select_config(int m, int n, int k, int ptr_align)
     for (size_t i = 0; g_table[i].config; ++i)
         if (g_table[i].m == m && g_table[i].n == n && g_table[i].k == k && resolved[i] >= 0 &&
             config_supports(resolved[i], m, n, k, ptr_align))
-            return {resolved[i], g_table[i].group_m, g_table[i].ksplit > 0 ? g_table[i].ksplit : 1};
+            return {resolved[i], g_table[i].group_m, g_table[i].ksplit > 0 ? g_table[i].ksplit : 1, g_table[i].spread};
     return heuristic(m, n, k, ptr_align);
 }
 
@@ -319,6 +321,7 @@ QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n
         ch.cfg = cfg & 0xFFFF;
         ch.group_m = (cfg >> 16) & 0xFF;
         ch.ksplit = (cfg >> 24) & 0x3F;
+        ch.spread = (cfg >> 30) & 1;
         if (ch.group_m == 0) ch.group_m = 4;
         if (ch.ksplit == 0) ch.ksplit = 1;
         if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
@@ -332,7 +335,7 @@ QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n
         const hipError_t ez = hipGetLastError();
         if (ez != hipSuccess) return fail_launch(ez);
     }
-    const hipError_t e = g_configs[ch.cfg].launch(p, s, ch.group_m | (ch.ksplit << 8));
+    const hipError_t e = g_configs[ch.cfg].launch(p, s, ch.group_m | (ch.ksplit << 8) | (ch.spread << 16));
     return e == hipSuccess ? QM_OK : fail_launch(e);
 }
 
@@ -345,7 +348,7 @@ QM_EXPORT int qm_select_config(int m, int n, int k, int ptr_align)
 {
     if (m < 1 || n < 1 || k < 2 || (k & 1)) return QM_ERR_SHAPE;
     const Choice ch = select_config(m, n, k, ptr_align);
-    return ch.cfg | (ch.group_m << 16) | (ch.ksplit << 24);
+    return ch.cfg | (ch.group_m << 16) | (ch.ksplit << 24) | (ch.spread << 30);
 }
 
 QM_EXPORT int qm_num_configs(void) { return g_num_configs; }

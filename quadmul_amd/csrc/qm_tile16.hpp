@@ -54,6 +54,28 @@ __device__ __forceinline__ void mfma16_settle(v4i &acc)
     asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc));
 }
 
+// A use of `x` that generates no code: the value has to exist at this point of the program.
+__device__ __forceinline__ void keep_here(const v4i &x) { asm volatile("" ::"v"(x)); }
+
+// One accumulator register -> ordinary register.  Inside the loop the accumulators are
+// touched by asm statements only: an ordinary read there makes the register allocator
+// treat them as general values, and it starts moving and spilling them.
+__device__ __forceinline__ int acc_read(const int acc_elem)
+{
+    int dst;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(dst) : "a"(acc_elem));
+    return dst;
+}
+
+// acc = 0, as an MFMA on zero operands with a zero addend.  The accumulators are only
+// ever redefined by asm statements that tie them in place; an ordinary assignment here
+// would give the register allocator a second, unrelated definition to merge at the loop
+// head, which it does by copying all of them.
+__device__ __forceinline__ void mfma16_zero(v4i &acc, const v4i &zero)
+{
+    asm volatile("s_nop 1\n\tv_mfma_i32_16x16x64_i8 %0, %1, %1, 0" : "+a"(acc) : "v"(zero));
+}
+
 template <int BM_, int BN_, int WGM_, int WGN_, int STAGES_ = 4, int OCC_ = 1>
 struct Tile16Cfg {
     static constexpr int OCC = OCC_;  // workgroups meant to share a CU (sets the register budget)
@@ -92,59 +114,97 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     const int wm = wave / Cfg::WGN, wn = wave % Cfg::WGN;
     const int r = lane & 15, g = lane >> 4;
 
-    // workgroup -> (K split, tile): XCD-contiguous id, tiles in columns of group_m
-    const int gid = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    // ---- work items ----
+    // An item is one (K split, output tile) pair.  The grid is persistent: workgroup w runs
+    // items w, w + G, w + 2G, ... (G = gridDim.x, at most the number of items) as ONE
+    // continuous stream of K-steps, so the loads of the next item's first tiles are already
+    // in flight while the current item finishes and its result is stored.  G is a multiple
+    // of 8 whenever a workgroup gets more than one item, so an item's index modulo 8 is the
+    // XCD it runs on and the XCD-contiguous renumbering applies to items as it would to
+    // workgroups of a one-item-per-workgroup launch.
+    const int G = gridDim.x;
     const int ntiles = tiles_m * tiles_n;
-    // (readfirstlane: the quotient is computed on the vector ALU; everything derived from it
-    // is wave-uniform and belongs in scalar registers)
-    const int ks = __builtin_amdgcn_readfirstlane(gid / ntiles), pid = gid - ks * ntiles;
-    const int width = group_m * tiles_n;
-    const int first_m = (pid / width) * group_m;
-    const int gsz = min(tiles_m - first_m, group_m);
-    const int m0 = __builtin_amdgcn_readfirstlane((first_m + (pid % width) % gsz) * BM);
-    const int n0 = __builtin_amdgcn_readfirstlane(((pid % width) / gsz) * BN);
-
-    // This workgroup contracts K-steps [kt0, kt0 + KT) of the K / 128 in total (all of
-    // them unless the launch splits K; then the partial sums meet in C by atomic adds
-    // and the host has zero-filled C beforehand).
+    const int nitems = ntiles * ksplit;
     const int Kb = p.K >> 1;
     const int kt_all = p.K / BK;  // K is a multiple of 128 for this kernel
     const int kps = (kt_all + ksplit - 1) / ksplit;
-    const int kt0 = __builtin_amdgcn_readfirstlane(min(ks * kps, kt_all - 1));
-    const int KT = __builtin_amdgcn_readfirstlane(min(kps, kt_all - ks * kps));  // >= 1: the launcher never creates an empty split
-    // (no early exit here: a branch around the whole body costs the register allocator
-    // dearly; an empty split would simply run no K-step and add zeros)
+
+    // item -> tile origin and K-step range [kt0, kt0 + KT); KT >= 1 (the launcher never
+    // creates an empty split).  Tiles are numbered in columns of group_m.
+    // (readfirstlane: the quotients are computed on the vector ALU; everything derived from
+    // them is wave-uniform and belongs in scalar registers)
+    auto locate = [&](const int item, int &m0, int &n0, int &kt0, int &KT) {
+        const int gid = xcd_contiguous_id(item, nitems);
+        const int ks = __builtin_amdgcn_readfirstlane(gid / ntiles), pid = gid - ks * ntiles;
+        const int width = group_m * tiles_n;
+        const int first_m = (pid / width) * group_m;
+        const int gsz = min(tiles_m - first_m, group_m);
+        m0 = __builtin_amdgcn_readfirstlane((first_m + (pid % width) % gsz) * BM);
+        n0 = __builtin_amdgcn_readfirstlane(((pid % width) / gsz) * BN);
+        kt0 = __builtin_amdgcn_readfirstlane(min(ks * kps, kt_all - 1));
+        KT = __builtin_amdgcn_readfirstlane(max(min(kps, kt_all - ks * kps), 1));
+    };
 
     // ---- global -> LDS: piece q of this wave covers tile rows (q*WAVES + wave)*16 .. +15.
     // The hardware puts lane l's 16 bytes at (wave-uniform LDS base) + 16*l, i.e. row l/4,
     // physical chunk l%4 of the piece; the lane therefore fetches the logical chunk that
     // the swizzle (chunk ^ ((row >> 1) & 3)) maps there.  Rows past the edge of the matrix
     // are clamped (their products are never stored).
+    //
+    // The loads run AHEAD K-steps in front of the MFMAs, through item boundaries, so they
+    // have a cursor of their own: (item, K-step within the item) and the per-lane row
+    // offsets of that item's tile.  Every item is padded to an even number of K-steps (the
+    // padding step re-reads the last real tile; its products are masked to zero).
     const int dma_row = lane >> 2;
     const int dma_ch = (lane & 3) ^ ((dma_row >> 1) & 3);
     uint32_t a_goff[A_PIECES], b_goff[B_PIECES];
+    int d_item = blockIdx.x, d_kt = 0, d_kt0, d_KT;
+    // (scalar part first: only dma_base stays live in a vector register between items)
+    const int dma_base = wave * 16 + dma_row;
+    const uint32_t dma_col = dma_ch * 16;
+    auto cursor_load = [&]() {
+        int m0, n0;
+        locate(d_item, m0, n0, d_kt0, d_KT);
 #pragma unroll
-    for (int q = 0; q < A_PIECES; ++q)
-        a_goff[q] = (uint32_t)min(m0 + (q * WAVES + wave) * 16 + dma_row, p.M - 1) * (uint32_t)Kb + dma_ch * 16;
+        for (int q = 0; q < A_PIECES; ++q)
+            a_goff[q] = (uint32_t)min((m0 + q * WAVES * 16) + dma_base, p.M - 1) * (uint32_t)Kb + dma_col;
 #pragma unroll
-    for (int q = 0; q < B_PIECES; ++q)
-        b_goff[q] = (uint32_t)min(n0 + (q * WAVES + wave) * 16 + dma_row, p.N - 1) * (uint32_t)Kb + dma_ch * 16;
+        for (int q = 0; q < B_PIECES; ++q)
+            b_goff[q] = (uint32_t)min((n0 + q * WAVES * 16) + dma_base, p.N - 1) * (uint32_t)Kb + dma_col;
+    };
+    const uint8_t *a_src, *b_src;  // operand base + K offset of the step the cursor points at
+    auto cursor_point = [&]() {
+        const int kofs = (d_kt0 + min(d_kt, d_KT - 1)) * (BK / 2);
+        a_src = p.A + kofs;
+        b_src = p.B + kofs;
+    };
+    // Past the last item the cursor stays on the last step: those loads land in stages
+    // nobody reads any more.
+    auto cursor_advance = [&]() {
+        ++d_kt;
+        if (d_kt >= d_KT + (d_KT & 1)) {
+            if (d_item + G < nitems) {
+                d_item += G;
+                d_kt = 0;
+                cursor_load();
+            } else {
+                d_kt = d_KT - 1;
+            }
+        }
+        cursor_point();
+    };
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t dma_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 16 * PITCH);
 
-    // piece index -> (operand, piece): issues one wave-wide load of tile `kt` into `stage_byte`.
-    // Tiles past the end re-read the last tile; they land in a stage nobody reads any more.
-    auto dma_piece = [&](int piece, int stage_byte, int kt) {
-        const int kofs = (kt0 + max(min(kt, KT - 1), 0)) * (BK / 2);
+    // piece index -> (operand, piece): one wave-wide load of the cursor's step into `stage_byte`
+    auto dma_piece = [&](int piece, int stage_byte) {
         if (piece < A_PIECES) {
             const uint32_t dst = dma_lds + stage_byte + piece * WAVES * 16 * PITCH;
-            const uint8_t *src = p.A + kofs;
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(a_goff[piece]), "s"(src) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(a_goff[piece]), "s"(a_src) : "memory", "m0");
         } else {
             const int b = piece - A_PIECES;
             const uint32_t dst = dma_lds + stage_byte + Cfg::A_BYTES + b * WAVES * 16 * PITCH;
-            const uint8_t *src = p.B + kofs;
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(b_goff[b]), "s"(src) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(b_goff[b]), "s"(b_src) : "memory", "m0");
         }
     };
 
@@ -168,16 +228,21 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 
-    // ---- prologue: tiles 0 .. STAGES-2 on their way into stages 0 .. STAGES-2; wait for 0 and 1 ----
-    constexpr int STAGES = Cfg::STAGES, AHEAD = STAGES - 1;  // tile kt+AHEAD is issued during K-step kt
+    // ---- prologue: steps 0 .. STAGES-2 of the stream on their way into stages 0 .. STAGES-2;
+    // wait for 0 and 1 ----
+    constexpr int STAGES = Cfg::STAGES, AHEAD = STAGES - 1;  // step s+AHEAD is issued during step s
+    cursor_load();
+    cursor_point();
 #pragma unroll
-    for (int t = 0; t < AHEAD; ++t)
+    for (int t = 0; t < AHEAD; ++t) {
 #pragma unroll
-        for (int q = 0; q < NP; ++q) dma_piece(q, t * STAGE, t);
+        for (int q = 0; q < NP; ++q) dma_piece(q, t * STAGE);
+        cursor_advance();
+    }
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 2) * NP) : "memory");
     __syncthreads();
 
-    // B fragments of the current tile (widened) and of the next (being widened); the two
+    // B fragments of the current step (widened) and of the next (being widened); the two
     // sets swap roles every K-step, so the K loop is unrolled by two.  A: ping-pong per
     // sub-step (FM is even, so the parity carries over K-steps).
     v4i b_ev[2][FN], b_od[2][FN], b_pk[2];
@@ -187,7 +252,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     x16_expand(read_a(0, 0), a_ev[0], a_od[0]);
     a_pk[1] = read_a(0, 1);
 
-    // byte offsets of the ring stages: tile kt, kt+1, ..., and the one being (re)filled
+    // byte offsets of the ring stages: step s, s+1, ..., and the one being (re)filled
     int ring[STAGES];
 #pragma unroll
     for (int t = 0; t < STAGES; ++t) ring[t] = t * STAGE;
@@ -206,14 +271,14 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     uint32_t amask;
     asm volatile("s_mov_b32 %0, 0xf0f0f0f0" : "=s"(amask));
 
-    auto k_step = [&](const int kt, auto bs_tag) {
-        constexpr int bs = decltype(bs_tag)::value;  // B register set holding tile kt
+    // One K-step: contracts the step in ring[0] (its B fragments sit widened in register set
+    // bs), reads and widens the B fragments of the step in ring[1] with `bmask` (zero when
+    // that step is an item's padding), and issues the cursor's loads into the last stage.
+    auto k_step = [&](const uint32_t bmask, auto bs_tag) {
+        constexpr int bs = decltype(bs_tag)::value;
         constexpr int SLOTS = 2 * FN;                // MFMAs per sub-step
         constexpr int BSHARE = 12 * FN / FM;         // B widening ops per sub-step
         constexpr int NOPS = 12 + BSHARE;            // VALU ops per sub-step, spread over slots 1..SLOTS-1
-        // The loop runs K-steps in pairs; when the number of tiles is odd the last step
-        // contracts a tile that does not exist, so its B operand is widened to zero.
-        const uint32_t bmask = kt + 1 < KT ? amask : 0u;
         static_for<0, FM>([&](auto i_) {
             constexpr int i = decltype(i_)::value;
             constexpr int pa = i & 1;
@@ -223,7 +288,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 if constexpr (s < FN) mfma16_acc(acc[i][s], b_ev[bs][s], a_ev[pa]);
                 else mfma16_acc(acc[i][s - FN], b_od[bs][s - FN], a_od[pa]);
                 if constexpr (s == 0) {
-                    // -- LDS reads: B fragments of tile kt+1 whose widening starts in this
+                    // -- LDS reads: B fragments of the next step whose widening starts in this
                     //    sub-step, and the A fragment two sub-steps ahead --
                     static_for<0, FN>([&](auto j_) {
                         constexpr int j = decltype(j_)::value;
@@ -233,7 +298,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     a_pk[pa] = read_a(i2 >= FM ? ring[1] : ring[0], i2 % FM);
                 } else {
                     // -- this slot's share of the widening work: ops [lo, hi) of the sub-step's
-                    //    list: 12 ops for the next A fragment, then BSHARE ops of B(kt+1) --
+                    //    list: 12 ops for the next A fragment, then BSHARE ops of the next B --
                     constexpr int lo = (s - 1) * NOPS / (SLOTS - 1), hi = s * NOPS / (SLOTS - 1);
                     static_for<lo, hi>([&](auto o_) {
                         constexpr int o = decltype(o_)::value;
@@ -246,65 +311,107 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                         }
                     });
                 }
-                // -- DMA pieces of tile kt+3, one sub-step apart --
+                // -- DMA pieces of the step AHEAD of this one, one sub-step apart --
                 if constexpr (s == SLOTS - 1) {
                     static_for<0, NP>([&](auto q_) {
                         constexpr int q = decltype(q_)::value;
-                        if constexpr (q * FM / NP == i) dma_piece(q, ring[STAGES - 1], kt + AHEAD);
+                        if constexpr (q * FM / NP == i) dma_piece(q, ring[STAGES - 1]);
                     });
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
-        // Tile kt+2 must have landed, and every wave must be done reading tile kt's stage,
-        // before the roles rotate; the younger tiles stay in flight.
+        // (The fragments widened for the next step are only used after the branches of the
+        // load cursor below; without a use here the compiler sinks their widening out of
+        // the MFMA slots to the far side of those branches.)
+        static_for<0, FN>([&](auto j_) {
+            constexpr int j = decltype(j_)::value;
+            keep_here(b_ev[bs ^ 1][j]);
+            keep_here(b_od[bs ^ 1][j]);
+        });
+        keep_here(a_ev[0]);
+        keep_here(a_od[0]);
+        keep_here(a_pk[1]);
+        // The step two ahead must have landed, and every wave must be done reading this
+        // step's stage, before the roles rotate; the younger steps stay in flight.
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((AHEAD - 2) * NP) : "memory");
         const int t = ring[0];
 #pragma unroll
         for (int u = 0; u + 1 < STAGES; ++u) ring[u] = ring[u + 1];
         ring[STAGES - 1] = t;
+        cursor_advance();
     };
 
-    for (int kt = 0; kt < KT; kt += 2) {
-        k_step(kt, std::integral_constant<int, 0>{});
-        k_step(kt + 1, std::integral_constant<int, 1>{});
-    }
-    // Drain the DMA before the LDS is released, and let the last MFMAs retire before their
-    // accumulators are read: the compiler does not know the asm statements were MFMAs, so
-    // the wait is tied to the accumulators written last (it cannot be scheduled around).
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    static_for<(FN > 4 ? FN - 4 : 0), FN>([&](auto j_) {
-        mfma16_settle(acc[FM - 1][decltype(j_)::value]);
-    });
-
-    // ---- epilogue: drop the factor 256, guarded 16-byte stores ----
     const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
+    const int c_row = wm * Cfg::WM + r, c_col = wn * Cfg::WN + g * 4;  // this lane's place in a 16x16 block
+    int c_item = blockIdx.x, c_kt = 0, c_m0, c_n0, c_kt0, c_KT;
+    locate(c_item, c_m0, c_n0, c_kt0, c_KT);
+    for (;;) {
+        // K-steps in pairs; when the item has an odd number of them, the second of the last
+        // pair is the padding step and its B operand is widened to zero
+        // (the mask is made opaque: knowing it is either all-ones-per-nibble or zero, the
+        // compiler would hoist the whole widening of B out of the MFMA slots into a branch)
+        uint32_t bmask = c_kt + 1 < c_KT ? amask : 0u;
+        asm volatile("" : "+s"(bmask));
+        k_step(bmask, std::integral_constant<int, 0>{});
+        k_step(amask, std::integral_constant<int, 1>{});
+        c_kt += 2;
+        if (c_kt < c_KT) continue;
+
+        // ---- the item is complete: let the last MFMAs retire before their accumulators are
+        // read (the compiler does not know the asm statements were MFMAs, so the wait is tied
+        // to the accumulators written last and cannot be scheduled around) ----
+        static_for<(FN > 4 ? FN - 4 : 0), FN>([&](auto j_) {
+            mfma16_settle(acc[FM - 1][decltype(j_)::value]);
+        });
+        // ---- drop the factor 256, guarded 16-byte stores, clear the accumulators ----
+        v4i zero4;
+        asm volatile("v_mov_b32 %0, 0" : "=v"(zero4.x));  // (opaque, so the MFMA operand is a plain register tuple)
+        zero4.y = zero4.z = zero4.w = zero4.x;
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        const int m = m0 + wm * Cfg::WM + i * 16 + r;
-        if (m >= p.M) continue;
-        int32_t *crow = p.C + (size_t)m * p.N;
+        for (int i = 0; i < FM; ++i) {
+            const int m = (c_m0 + i * 16) + c_row;
+            int32_t *crow = p.C + (size_t)m * p.N;
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const int n = n0 + wn * Cfg::WN + j * 16 + g * 4;
-            v4i v = acc[i][j];
-            v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
-            if (ksplit > 1) {
-                // every partial accumulator is a multiple of 256, so the shifted partials add
-                // up to the shifted total; integer atomics make the order irrelevant
+            for (int j = 0; j < FN; ++j) {
+                const int n = (c_n0 + j * 16) + c_col;
+                v4i v;
+                v.x = acc_read(acc[i][j].x);
+                v.y = acc_read(acc[i][j].y);
+                v.z = acc_read(acc[i][j].z);
+                v.w = acc_read(acc[i][j].w);
+                mfma16_zero(acc[i][j], zero4);
+                if (m >= p.M) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    continue;
+                }
+                v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
+                if (ksplit > 1) {
+                    // every partial accumulator is a multiple of 256, so the shifted partials add
+                    // up to the shifted total; integer atomics make the order irrelevant
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            } else if (vec_ok && n + 3 < p.N) {
-                *reinterpret_cast<v4i *>(crow + n) = v;
-            } else {
-                if (n < p.N) crow[n] = v.x;
-                if (n + 1 < p.N) crow[n + 1] = v.y;
-                if (n + 2 < p.N) crow[n + 2] = v.z;
-                if (n + 3 < p.N) crow[n + 3] = v.w;
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else if (vec_ok && n + 3 < p.N) {
+                    *reinterpret_cast<v4i *>(crow + n) = v;
+                } else {
+                    if (n < p.N) crow[n] = v.x;
+                    if (n + 1 < p.N) crow[n + 1] = v.y;
+                    if (n + 2 < p.N) crow[n + 2] = v.z;
+                    if (n + 3 < p.N) crow[n + 3] = v.w;
+                }
+                // one block at a time: the widened fragments of the next step stay live
+                // across this code, so there are few registers to stage results in
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+        c_item += G;
+        if (c_item >= nitems) break;
+        locate(c_item, c_m0, c_n0, c_kt0, c_KT);
+        c_kt = 0;
     }
+    // drain the DMA before the LDS is released
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 }  // namespace qm

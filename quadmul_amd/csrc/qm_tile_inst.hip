@@ -26,12 +26,32 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
     return hipGetLastError();
 }
 
+// Pipelined kernel: opt additionally holds the K split in bits 8..15 (the caller has
+// zero-filled C when it is above 1) and, in bit 16, "one work item per workgroup".  By
+// default the grid is persistent: as many workgroups as the device holds at once, each
+// running several (K split, tile) items back to back.
 template <class Cfg, class Kernel>
-static hipError_t launch_tiled_splitk(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
+static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
 {
     static bool lds_ok[QM_MAX_DEVICES] = {};
+    static int resident[QM_MAX_DEVICES] = {};  // workgroups the device holds at once (0: not asked yet)
     hipError_t e = ensure_dynamic_lds(kernel, Cfg::LDS_BYTES, lds_ok);
     if (e != hipSuccess) return e;
+    int dev = 0;
+    e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= QM_MAX_DEVICES) return hipErrorInvalidDevice;
+    if (resident[dev] == 0) {
+        int per_cu = 0, cus = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, Cfg::THREADS, Cfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return e;
+        if (per_cu < 1) per_cu = 1;
+        // a multiple of 8, so that an item index modulo 8 names the XCD it runs on
+        int g = per_cu * cus / 8 * 8;
+        resident[dev] = g < 8 ? 8 : g;
+    }
     const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
     int group_m = opt & 0xFF, ksplit = (opt >> 8) & 0xFF;
     if (group_m < 1) group_m = 1;
@@ -42,7 +62,11 @@ static hipError_t launch_tiled_splitk(Kernel kernel, const GemmArgs &p, hipStrea
         const int kt = p.K / Cfg::BK, kps = (kt + ksplit - 1) / ksplit;
         ksplit = (kt + kps - 1) / kps;
     }
-    kernel<<<dim3(tiles_m * tiles_n * ksplit), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, tiles_m, tiles_n, group_m, ksplit);
+    const long long items = (long long)tiles_m * tiles_n * ksplit;
+    if (items > 0x7FFFFFFF) return hipErrorInvalidValue;
+    int grid = (int)items;
+    if (!(opt & 0x10000) && grid > resident[dev]) grid = resident[dev];
+    kernel<<<dim3(grid), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, tiles_m, tiles_n, group_m, ksplit);
     return hipGetLastError();
 }
 
@@ -61,7 +85,7 @@ static hipError_t launch_tiled_splitk(Kernel kernel, const GemmArgs &p, hipStrea
     hipError_t QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &p, hipStream_t s, int gm) \
     {                                                                                            \
         using Cfg = Tile16Cfg<BM, BN, WGM, WGN, ST, OCC>;                                        \
-        return launch_tiled_splitk<Cfg>(&gemm_tile16_kernel<Cfg>, p, s, gm);                   \
+        return launch_tiled_persistent<Cfg>(&gemm_tile16_kernel<Cfg>, p, s, gm);                   \
     }                                                                                   \
     }
 

@@ -255,6 +255,36 @@ def test_baseline_configs_full_compare(oracle_mod, row):
     assert oracle_mod.compare(got_d.cpu().numpy(), want) == -1
 
 
+# More tiles than the device holds workgroups: every persistent workgroup runs several
+# (K split, tile) items back to back, with 1, 2, 3 and 5 K-steps per item (the load
+# cursor crosses item boundaries inside the ring; odd counts exercise the padding step),
+# ragged edges, and the one-item-per-workgroup launch of the same configurations.
+PERSISTENT_SHAPES = [(4352, 4400, 128), (4400, 4352, 256), (4352, 4400, 384), (2500, 9000, 640)]
+
+
+@pytest.mark.parametrize("shape", PERSISTENT_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_persistent_grid_many_items_per_workgroup(oracle_mod, shape):
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 5000 + k)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    want_d = fp32_matmul_on_gpu(a, b)
+    rows = np.unique(np.concatenate([np.arange(0, m, 61), [m - 1, 255, 256, 257, 511, 512]])).astype(np.int32)
+    want_rows = oracle_mod.gemm_i4_rows(ap.numpy(), bp.numpy(), rows)
+    assert oracle_mod.compare(want_d.cpu().numpy()[rows], want_rows) == -1  # the fast check agrees with the oracle
+    ran = 0
+    for cfg, name in enumerate(qm.config_names()):
+        if not name.startswith("q") or not qm.config_supports(cfg, m, n, k):
+            continue
+        for gm, ks, spread in [(4, 1, 0), (1, 1, 0), (4, 1, 1), (3, 2, 0), (4, 3, 0), (2, 2, 1)]:
+            got_d = poisoned_c(m, n, DEV)
+            qm.gemm_cfg(a_d, b_d, got_d, m, n, k, cfg | (gm << 16) | (ks << 24) | (spread << 30))
+            torch.cuda.synchronize()
+            assert torch.equal(got_d, want_d), f"{name} group_m={gm} ksplit={ks} spread={spread}"
+        ran += 1
+    assert ran >= 4
+
+
 @pytest.mark.parametrize("row", [(8, 8192, 8192, 8192), (9, 8000, 8000, 8064)], ids=lambda r: "x".join(map(str, r[1:])))
 def test_large_configs(oracle_mod, row):
     i, m, n, k = row
