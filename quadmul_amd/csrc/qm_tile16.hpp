@@ -95,7 +95,7 @@ struct Tile16Cfg {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
     static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
     static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
-    static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
+    static_assert(FM >= 2 && FM % 2 == 0 && FN >= 2 && FN % 2 == 0, "pipeline needs an even number (>= 2) of A fragments per wave; the epilogue pairs B fragments");
     static_assert((12 * FN) % FM == 0, "B widening must split evenly over the sub-steps");
 };
 
@@ -343,7 +343,12 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     };
 
     const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
-    const int c_row = wm * Cfg::WM + r, c_col = wn * Cfg::WN + g * 4;  // this lane's place in a 16x16 block
+    // this lane's place in the 16 x 32 area of two neighbouring blocks, after the swap
+    const int c_row = wm * Cfg::WM + (r & 7), c_col = wn * Cfg::WN + ((r >> 3) << 4) + g * 4;
+    // byte offset of that place from the tile's corner (32 bits are enough for the rows of one
+    // tile when N is below 2^21), and whether C can take unguarded 16-byte stores at all
+    const uint32_t lane_c = ((uint32_t)c_row * (uint32_t)p.N + (uint32_t)c_col) * 4u;
+    const bool plain_c = vec_ok && ksplit == 1 && p.N < (1 << 21);
     int c_item = blockIdx.x, c_kt = 0, c_m0, c_n0, c_kt0, c_KT;
     locate(c_item, c_m0, c_n0, c_kt0, c_KT);
     for (;;) {
@@ -365,45 +370,76 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             mfma16_settle(acc[FM - 1][decltype(j_)::value]);
         });
         // ---- drop the factor 256, guarded 16-byte stores, clear the accumulators ----
+        // (the accumulators are cleared as they are read)
         v4i zero4;
         asm volatile("v_mov_b32 %0, 0" : "=v"(zero4.x));  // (opaque, so the MFMA operand is a plain register tuple)
         zero4.y = zero4.z = zero4.w = zero4.x;
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-            const int m = (c_m0 + i * 16) + c_row;
+        // A 16x16 block leaves the MFMA as 16 rows x 64 bytes per wave-wide store, and a
+        // CU pushes such half-line stores out more than three times slower than stores
+        // that cover whole 128-byte lines.  Two blocks that are neighbours along n hold,
+        // between them, 16 rows x 128 bytes; lanes r and r^8 (same 16-lane row of the
+        // wave) swap one block each, after which one store carries rows 0..7 and the
+        // next rows 8..15, both 128 bytes wide.
+        auto store_piece = [&](const int m, const int n, const v4i v) {
+            if (m >= p.M) return;
             int32_t *crow = p.C + (size_t)m * p.N;
+            if (ksplit > 1) {
+                // every partial accumulator is a multiple of 256, so the shifted partials add
+                // up to the shifted total; integer atomics make the order irrelevant
 #pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                const int n = (c_n0 + j * 16) + c_col;
-                v4i v;
-                v.x = acc_read(acc[i][j].x);
-                v.y = acc_read(acc[i][j].y);
-                v.z = acc_read(acc[i][j].z);
-                v.w = acc_read(acc[i][j].w);
-                mfma16_zero(acc[i][j], zero4);
-                if (m >= p.M) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    continue;
-                }
-                v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
-                if (ksplit > 1) {
-                    // every partial accumulator is a multiple of 256, so the shifted partials add
-                    // up to the shifted total; integer atomics make the order irrelevant
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                } else if (vec_ok && n + 3 < p.N) {
-                    *reinterpret_cast<v4i *>(crow + n) = v;
-                } else {
-                    if (n < p.N) crow[n] = v.x;
-                    if (n + 1 < p.N) crow[n + 1] = v.y;
-                    if (n + 2 < p.N) crow[n + 2] = v.z;
-                    if (n + 3 < p.N) crow[n + 3] = v.w;
-                }
-                // one block at a time: the widened fragments of the next step stay live
-                // across this code, so there are few registers to stage results in
-                __builtin_amdgcn_sched_barrier(0);
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else if (vec_ok && n + 3 < p.N) {
+                *reinterpret_cast<v4i *>(crow + n) = v;
+            } else {
+                if (n < p.N) crow[n] = v.x;
+                if (n + 1 < p.N) crow[n + 1] = v.y;
+                if (n + 2 < p.N) crow[n + 2] = v.z;
+                if (n + 3 < p.N) crow[n + 3] = v.w;
             }
+        };
+        // Whole tiles inside the matrix (the usual case) take a path without per-lane
+        // guards: with one wave per SIMD every instruction here is exposed, and the guarded
+        // version is several times longer.  (The accumulators must be read and cleared by
+        // ONE set of asm statements -- a second copy of them on another branch makes the
+        // register allocator merge 256 registers by copying -- so only the stores branch,
+        // and the guarded stores are marked unlikely to keep them out of the straight run.)
+        char *const tile_c = reinterpret_cast<char *>(p.C + ((size_t)c_m0 * p.N + c_n0));  // wave-uniform
+        const bool whole = plain_c && c_m0 + BM <= p.M && c_n0 + BN <= p.N;
+        {
+            static_for<0, FM>([&](auto i_) {
+                constexpr int i = decltype(i_)::value;
+                static_for<0, FN / 2>([&](auto jp_) {
+                    constexpr int j = 2 * decltype(jp_)::value;
+                    v4i x, y, lo, hi;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        x[e] = acc_read(acc[i][j][e]);
+                        y[e] = acc_read(acc[i][j + 1][e]);
+                    }
+                    mfma16_zero(acc[i][j], zero4);
+                    mfma16_zero(acc[i][j + 1], zero4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        // row_ror:8 pairs lane r with lane r^8; the bank mask picks the half that takes
+                        // its partner's value (banks 2,3 = r >= 8; banks 0,1 = r < 8), the rest keep theirs
+                        lo[e] = __builtin_amdgcn_update_dpp(x[e], y[e], 0x128, 0xF, 0xC, false) >> 8;
+                        hi[e] = __builtin_amdgcn_update_dpp(y[e], x[e], 0x128, 0xF, 0x3, false) >> 8;
+                    }
+                    if (__builtin_expect(whole, 1)) {
+                        char *const at = tile_c + ((size_t)(i * 16) * p.N + j * 16) * 4;  // wave-uniform
+                        *reinterpret_cast<v4i *>(at + lane_c) = lo;
+                        *reinterpret_cast<v4i *>(at + (size_t)p.N * 32 + lane_c) = hi;
+                    } else {
+                        const int m = (c_m0 + i * 16) + c_row, n = (c_n0 + j * 16) + c_col;
+                        store_piece(m, n, lo);
+                        store_piece(m + 8, n, hi);
+                    }
+                    // one pair at a time: the widened fragments of the next step stay live
+                    // across this code, so there are few registers to stage results in
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
         }
         c_item += G;
         if (c_item >= nitems) break;
