@@ -107,6 +107,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     constexpr int PITCH = Cfg::PITCH, STAGE = Cfg::STAGE_BYTES, WAVES = Cfg::WAVES;
     constexpr int A_PIECES = Cfg::A_PIECES, B_PIECES = Cfg::B_PIECES, NP = A_PIECES + B_PIECES;
 
+    // (Every lambda below is marked always_inline: the state they share -- accumulators,
+    // ring, load cursor -- lives in registers only as long as nothing is outlined.)
     extern __shared__ __align__(16) uint8_t smem[];
 
     const int tid = threadIdx.x;
@@ -133,14 +135,36 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // creates an empty split).  Tiles are numbered in columns of group_m.
     // (readfirstlane: the quotients are computed on the vector ALU; everything derived from
     // them is wave-uniform and belongs in scalar registers)
-    auto locate = [&](const int item, int &m0, int &n0, int &kt0, int &KT) {
-        const int gid = xcd_contiguous_id(item, nitems);
-        const int ks = __builtin_amdgcn_readfirstlane(gid / ntiles), pid = gid - ks * ntiles;
-        const int width = group_m * tiles_n;
+    //
+    // Items come in two ranges.  [0, nwhole): tiles that lie wholly inside the matrix, when C
+    // takes plain 16-byte stores and K is not split -- their write-out needs no guards and is
+    // folded into the last K-step.  [nwhole, nitems): everything else (the ragged right
+    // column and bottom row of tiles; or all items, when nwhole is 0), written out by the
+    // guarded code after the last K-step.  A workgroup's items ascend, so it runs its whole
+    // tiles first and then the rest: two loops one after the other.
+    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
+    const bool plain_c = vec_ok && ksplit == 1 && p.N < (1 << 21);
+    const int full_m = p.M / BM, full_n = p.N / BN;
+    const int nwhole = __builtin_amdgcn_readfirstlane(plain_c ? full_m * full_n : 0);
+    auto locate = [&](const int item, int &m0, int &n0, int &kt0, int &KT) __attribute__((always_inline)) {
+        // (both numberings are evaluated and one is picked: a branch here, with quotients
+        // from the vector ALU on one side only, costs the scalar registers of everything
+        // computed after it)
+        const int rows = nwhole ? full_m : tiles_m, cols = nwhole ? full_n : tiles_n;
+        const int gid = xcd_contiguous_id(nwhole ? min(item, nwhole - 1) : item, nwhole ? nwhole : nitems);
+        const int ks = __builtin_amdgcn_readfirstlane(gid / ntiles);  // 0 unless K is split (then nwhole is 0)
+        const int pid = gid - ks * ntiles;
+        const int width = group_m * cols;
         const int first_m = (pid / width) * group_m;
-        const int gsz = min(tiles_m - first_m, group_m);
-        m0 = __builtin_amdgcn_readfirstlane((first_m + (pid % width) % gsz) * BM);
-        n0 = __builtin_amdgcn_readfirstlane(((pid % width) / gsz) * BN);
+        const int gsz = min(rows - first_m, group_m);
+        const int tm_a = __builtin_amdgcn_readfirstlane(first_m + (pid % width) % gsz);
+        const int tn_a = __builtin_amdgcn_readfirstlane((pid % width) / gsz);
+        // ragged tiles: the right column top to bottom (if N is ragged), then the bottom row
+        const int e = item - nwhole, right = tiles_n > full_n ? tiles_m : 0;
+        const int tm_b = e < right ? e : full_m, tn_b = e < right ? full_n : e - right;
+        const bool ragged = nwhole != 0 && item >= nwhole;
+        m0 = (ragged ? tm_b : tm_a) * BM;
+        n0 = (ragged ? tn_b : tn_a) * BN;
         kt0 = __builtin_amdgcn_readfirstlane(min(ks * kps, kt_all - 1));
         KT = __builtin_amdgcn_readfirstlane(max(min(kps, kt_all - ks * kps), 1));
     };
@@ -162,7 +186,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // (scalar part first: only dma_base stays live in a vector register between items)
     const int dma_base = wave * 16 + dma_row;
     const uint32_t dma_col = dma_ch * 16;
-    auto cursor_load = [&]() {
+    auto cursor_load = [&]() __attribute__((always_inline)) {
         int m0, n0;
         locate(d_item, m0, n0, d_kt0, d_KT);
 #pragma unroll
@@ -173,14 +197,14 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             b_goff[q] = (uint32_t)min((n0 + q * WAVES * 16) + dma_base, p.N - 1) * (uint32_t)Kb + dma_col;
     };
     const uint8_t *a_src, *b_src;  // operand base + K offset of the step the cursor points at
-    auto cursor_point = [&]() {
+    auto cursor_point = [&]() __attribute__((always_inline)) {
         const int kofs = (d_kt0 + min(d_kt, d_KT - 1)) * (BK / 2);
         a_src = p.A + kofs;
         b_src = p.B + kofs;
     };
     // Past the last item the cursor stays on the last step: those loads land in stages
     // nobody reads any more.
-    auto cursor_advance = [&]() {
+    auto cursor_advance = [&]() __attribute__((always_inline)) {
         ++d_kt;
         if (d_kt >= d_KT + (d_KT & 1)) {
             if (d_item + G < nitems) {
@@ -197,7 +221,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     const uint32_t dma_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * 16 * PITCH);
 
     // piece index -> (operand, piece): one wave-wide load of the cursor's step into `stage_byte`
-    auto dma_piece = [&](int piece, int stage_byte) {
+    auto dma_piece = [&](int piece, int stage_byte) __attribute__((always_inline)) {
         if (piece < A_PIECES) {
             const uint32_t dst = dma_lds + stage_byte + piece * WAVES * 16 * PITCH;
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(a_goff[piece]), "s"(a_src) : "memory", "m0");
@@ -271,11 +295,87 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     uint32_t amask;
     asm volatile("s_mov_b32 %0, 0xf0f0f0f0" : "=s"(amask));
 
+    // ---- writing a finished tile ----
+    // A 16x16 block leaves the MFMA as 16 rows x 64 bytes per wave-wide store, and a CU
+    // pushes such half-line stores out more than three times slower than stores that
+    // cover whole 128-byte lines.  Two blocks that are neighbours along n hold, between
+    // them, 16 rows x 128 bytes; lanes r and r^8 (same 16-lane row of the wave) swap one
+    // block each, after which one store carries rows 0..7 and the next rows 8..15, both
+    // 128 bytes wide.
+    // this lane's place in the 16 x 32 area of two neighbouring blocks, after the swap
+    const int c_row = wm * Cfg::WM + (r & 7), c_col = wn * Cfg::WN + ((r >> 3) << 4) + g * 4;
+    // byte offset of that place from the tile's corner (32 bits are enough for the rows of one
+    // tile when N is below 2^21)
+    const uint32_t lane_c = ((uint32_t)c_row * (uint32_t)p.N + (uint32_t)c_col) * 4u;
+    int c_item = blockIdx.x, c_kt = 0, c_m0, c_n0, c_kt0, c_KT;  // the item being contracted
+    char *tile_c = nullptr;  // its corner in C (wave-uniform)
+    auto store_piece = [&](const int m, const int n, const v4i v) __attribute__((always_inline)) {
+        if (m >= p.M) return;
+        int32_t *crow = p.C + (size_t)m * p.N;
+        if (ksplit > 1) {
+            // every partial accumulator is a multiple of 256, so the shifted partials add
+            // up to the shifted total; integer atomics make the order irrelevant
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else if (vec_ok && n + 3 < p.N) {
+            *reinterpret_cast<v4i *>(crow + n) = v;
+        } else {
+            if (n < p.N) crow[n] = v.x;
+            if (n + 1 < p.N) crow[n + 1] = v.y;
+            if (n + 2 < p.N) crow[n + 2] = v.z;
+            if (n + 3 < p.N) crow[n + 3] = v.w;
+        }
+    };
+    v4i zero4;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(zero4.x));  // (opaque, so the MFMA operand is a plain register tuple)
+    zero4.y = zero4.z = zero4.w = zero4.x;
+    // The work for blocks (ib, j) and (ib, j+1), in four parts so that it can ride in four
+    // MFMA slots: read one block; read the other and clear both (the accumulators are only
+    // touched through asm statements: an ordinary read or write inside the loop makes the
+    // register allocator treat them as general values and copy them around); swap, drop
+    // the factor 256 and store rows 0..7; the same for rows 8..15.  `whole`: the tile lies
+    // inside the matrix and the stores need no guards (and no branches, which would cut
+    // the slot-by-slot schedule of a K-step apart).
+    v4i ex, ey;
+    auto write_part = [&](auto whole_, auto ib_, auto j_, auto q_) __attribute__((always_inline)) {
+        constexpr bool whole = decltype(whole_)::value;
+        constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value, q = decltype(q_)::value;
+        if constexpr (q == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ex[e] = acc_read(acc[ib][j][e]);
+        } else if constexpr (q == 1) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ey[e] = acc_read(acc[ib][j + 1][e]);
+            mfma16_zero(acc[ib][j], zero4);
+            mfma16_zero(acc[ib][j + 1], zero4);
+        } else {
+            // row_ror:8 pairs lane r with lane r^8; the bank mask picks the half that takes its
+            // partner's value (banks 2,3 = r >= 8; banks 0,1 = r < 8), the rest keep theirs
+            v4i v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                v[e] = (q == 2 ? __builtin_amdgcn_update_dpp(ex[e], ey[e], 0x128, 0xF, 0xC, false)
+                               : __builtin_amdgcn_update_dpp(ey[e], ex[e], 0x128, 0xF, 0x3, false)) >> 8;
+            constexpr int row = ib * 16 + (q == 2 ? 0 : 8);
+            if constexpr (whole) {
+                char *const at = tile_c + ((size_t)row * p.N + j * 16) * 4;  // wave-uniform
+                *reinterpret_cast<v4i *>(at + lane_c) = v;
+            } else {
+                store_piece((c_m0 + row) + c_row, (c_n0 + j * 16) + c_col, v);
+            }
+        }
+    };
+
     // One K-step: contracts the step in ring[0] (its B fragments sit widened in register set
     // bs), reads and widens the B fragments of the step in ring[1] with `bmask` (zero when
     // that step is an item's padding), and issues the cursor's loads into the last stage.
-    auto k_step = [&](const uint32_t bmask, auto bs_tag) {
+    // In the last step of a whole tile, row i-1 of the accumulator blocks is final once
+    // sub-step i begins: its write-out rides in the slots of sub-step i, two blocks per four
+    // slots, instead of stalling the matrix cores afterwards (row FM-1 is left to the caller).
+    auto k_step = [&](const uint32_t bmask, auto bs_tag, auto last_tag) __attribute__((always_inline)) {
         constexpr int bs = decltype(bs_tag)::value;
+        constexpr bool last = decltype(last_tag)::value;
         constexpr int SLOTS = 2 * FN;                // MFMAs per sub-step
         constexpr int BSHARE = 12 * FN / FM;         // B widening ops per sub-step
         constexpr int NOPS = 12 + BSHARE;            // VALU ops per sub-step, spread over slots 1..SLOTS-1
@@ -311,6 +411,10 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                         }
                     });
                 }
+                // -- write-out of the accumulator row finished one sub-step ago --
+                if constexpr (last && i >= 1)
+                    write_part(std::true_type{}, std::integral_constant<int, i - 1>{}, std::integral_constant<int, 2 * (s / 4)>{},
+                               std::integral_constant<int, s % 4>{});
                 // -- DMA pieces of the step AHEAD of this one, one sub-step apart --
                 if constexpr (s == SLOTS - 1) {
                     static_for<0, NP>([&](auto q_) {
@@ -333,8 +437,12 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         keep_here(a_od[0]);
         keep_here(a_pk[1]);
         // The step two ahead must have landed, and every wave must be done reading this
-        // step's stage, before the roles rotate; the younger steps stay in flight.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((AHEAD - 2) * NP) : "memory");
+        // step's stage, before the roles rotate; the younger steps stay in flight.  The
+        // counter also counts the stores of a last step, which are younger than the loads
+        // that must have landed: they are allowed to stay in flight as well (the counter
+        // cannot express more than 63).
+        constexpr int pending = (AHEAD - 2) * NP + (last ? (FM - 1) * FN : 0);
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(pending > 63 ? 63 : pending) : "memory");
         const int t = ring[0];
 #pragma unroll
         for (int u = 0; u + 1 < STAGES; ++u) ring[u] = ring[u + 1];
@@ -342,110 +450,41 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         cursor_advance();
     };
 
-    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
-    // this lane's place in the 16 x 32 area of two neighbouring blocks, after the swap
-    const int c_row = wm * Cfg::WM + (r & 7), c_col = wn * Cfg::WN + ((r >> 3) << 4) + g * 4;
-    // byte offset of that place from the tile's corner (32 bits are enough for the rows of one
-    // tile when N is below 2^21), and whether C can take unguarded 16-byte stores at all
-    const uint32_t lane_c = ((uint32_t)c_row * (uint32_t)p.N + (uint32_t)c_col) * 4u;
-    const bool plain_c = vec_ok && ksplit == 1 && p.N < (1 << 21);
-    int c_item = blockIdx.x, c_kt = 0, c_m0, c_n0, c_kt0, c_KT;
-    locate(c_item, c_m0, c_n0, c_kt0, c_KT);
-    for (;;) {
-        // K-steps in pairs; when the item has an odd number of them, the second of the last
-        // pair is the padding step and its B operand is widened to zero
+    // One item: K-steps in pairs; when the item has an odd number of them, the second of the
+    // last pair is the padding step and its B operand is widened to zero.
+    auto run_item = [&](auto whole_) __attribute__((always_inline)) {
+        constexpr bool whole = decltype(whole_)::value;
+        locate(c_item, c_m0, c_n0, c_kt0, c_KT);
+        for (c_kt = 0; c_kt + 2 < c_KT; c_kt += 2) {
+            k_step(amask, std::integral_constant<int, 0>{}, std::false_type{});
+            k_step(amask, std::integral_constant<int, 1>{}, std::false_type{});
+        }
         // (the mask is made opaque: knowing it is either all-ones-per-nibble or zero, the
         // compiler would hoist the whole widening of B out of the MFMA slots into a branch)
         uint32_t bmask = c_kt + 1 < c_KT ? amask : 0u;
         asm volatile("" : "+s"(bmask));
-        k_step(bmask, std::integral_constant<int, 0>{});
-        k_step(amask, std::integral_constant<int, 1>{});
-        c_kt += 2;
-        if (c_kt < c_KT) continue;
-
-        // ---- the item is complete: let the last MFMAs retire before their accumulators are
-        // read (the compiler does not know the asm statements were MFMAs, so the wait is tied
-        // to the accumulators written last and cannot be scheduled around) ----
+        tile_c = reinterpret_cast<char *>(p.C + ((size_t)c_m0 * p.N + c_n0));
+        k_step(bmask, std::integral_constant<int, 0>{}, std::false_type{});
+        k_step(amask, std::integral_constant<int, 1>{}, std::integral_constant<bool, whole>{});
+        // Let the last MFMAs retire before their accumulators are read (the compiler does not
+        // know the asm statements were MFMAs, so the wait is tied to the accumulators written
+        // last and cannot be scheduled around); then the rows not written out yet.
         static_for<(FN > 4 ? FN - 4 : 0), FN>([&](auto j_) {
             mfma16_settle(acc[FM - 1][decltype(j_)::value]);
         });
-        // ---- drop the factor 256, guarded 16-byte stores, clear the accumulators ----
-        // (the accumulators are cleared as they are read)
-        v4i zero4;
-        asm volatile("v_mov_b32 %0, 0" : "=v"(zero4.x));  // (opaque, so the MFMA operand is a plain register tuple)
-        zero4.y = zero4.z = zero4.w = zero4.x;
-        // A 16x16 block leaves the MFMA as 16 rows x 64 bytes per wave-wide store, and a
-        // CU pushes such half-line stores out more than three times slower than stores
-        // that cover whole 128-byte lines.  Two blocks that are neighbours along n hold,
-        // between them, 16 rows x 128 bytes; lanes r and r^8 (same 16-lane row of the
-        // wave) swap one block each, after which one store carries rows 0..7 and the
-        // next rows 8..15, both 128 bytes wide.
-        auto store_piece = [&](const int m, const int n, const v4i v) {
-            if (m >= p.M) return;
-            int32_t *crow = p.C + (size_t)m * p.N;
-            if (ksplit > 1) {
-                // every partial accumulator is a multiple of 256, so the shifted partials add
-                // up to the shifted total; integer atomics make the order irrelevant
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            } else if (vec_ok && n + 3 < p.N) {
-                *reinterpret_cast<v4i *>(crow + n) = v;
-            } else {
-                if (n < p.N) crow[n] = v.x;
-                if (n + 1 < p.N) crow[n + 1] = v.y;
-                if (n + 2 < p.N) crow[n + 2] = v.z;
-                if (n + 3 < p.N) crow[n + 3] = v.w;
-            }
-        };
-        // Whole tiles inside the matrix (the usual case) take a path without per-lane
-        // guards: with one wave per SIMD every instruction here is exposed, and the guarded
-        // version is several times longer.  (The accumulators must be read and cleared by
-        // ONE set of asm statements -- a second copy of them on another branch makes the
-        // register allocator merge 256 registers by copying -- so only the stores branch,
-        // and the guarded stores are marked unlikely to keep them out of the straight run.)
-        char *const tile_c = reinterpret_cast<char *>(p.C + ((size_t)c_m0 * p.N + c_n0));  // wave-uniform
-        const bool whole = plain_c && c_m0 + BM <= p.M && c_n0 + BN <= p.N;
-        {
-            static_for<0, FM>([&](auto i_) {
-                constexpr int i = decltype(i_)::value;
-                static_for<0, FN / 2>([&](auto jp_) {
-                    constexpr int j = 2 * decltype(jp_)::value;
-                    v4i x, y, lo, hi;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        x[e] = acc_read(acc[i][j][e]);
-                        y[e] = acc_read(acc[i][j + 1][e]);
-                    }
-                    mfma16_zero(acc[i][j], zero4);
-                    mfma16_zero(acc[i][j + 1], zero4);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        // row_ror:8 pairs lane r with lane r^8; the bank mask picks the half that takes
-                        // its partner's value (banks 2,3 = r >= 8; banks 0,1 = r < 8), the rest keep theirs
-                        lo[e] = __builtin_amdgcn_update_dpp(x[e], y[e], 0x128, 0xF, 0xC, false) >> 8;
-                        hi[e] = __builtin_amdgcn_update_dpp(y[e], x[e], 0x128, 0xF, 0x3, false) >> 8;
-                    }
-                    if (__builtin_expect(whole, 1)) {
-                        char *const at = tile_c + ((size_t)(i * 16) * p.N + j * 16) * 4;  // wave-uniform
-                        *reinterpret_cast<v4i *>(at + lane_c) = lo;
-                        *reinterpret_cast<v4i *>(at + (size_t)p.N * 32 + lane_c) = hi;
-                    } else {
-                        const int m = (c_m0 + i * 16) + c_row, n = (c_n0 + j * 16) + c_col;
-                        store_piece(m, n, lo);
-                        store_piece(m + 8, n, hi);
-                    }
-                    // one pair at a time: the widened fragments of the next step stay live
-                    // across this code, so there are few registers to stage results in
-                    __builtin_amdgcn_sched_barrier(0);
+        static_for<(whole ? FM - 1 : 0), FM>([&](auto ib_) {
+            static_for<0, FN / 2>([&](auto jp_) {
+                static_for<0, 4>([&](auto q_) {
+                    write_part(whole_, ib_, std::integral_constant<int, 2 * decltype(jp_)::value>{}, q_);
                 });
+                // one pair at a time: the widened fragments of the next step stay live
+                // across this code, so there are few registers to stage results in
+                __builtin_amdgcn_sched_barrier(0);
             });
-        }
-        c_item += G;
-        if (c_item >= nitems) break;
-        locate(c_item, c_m0, c_n0, c_kt0, c_KT);
-        c_kt = 0;
-    }
+        });
+    };
+    for (; c_item < nwhole; c_item += G) run_item(std::true_type{});
+    for (; c_item < nitems; c_item += G) run_item(std::false_type{});
     // drain the DMA before the LDS is released
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
