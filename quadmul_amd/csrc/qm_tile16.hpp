@@ -87,7 +87,14 @@ struct Tile16Cfg {
     static constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int STAGES = STAGES_;  // LDS ring depth: 4, or 5 for one more K-step of DMA latency cover
-    static constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+    static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+    // Per-wave LDS area through which finished accumulator blocks are turned into row-major
+    // order before they are stored: 16 rows x 64 int32, rows padded by 16 bytes so that the
+    // 16 lanes of a ds_write_b128 (one row each) fall into different banks.  Used when it
+    // fits beside the ring of every co-resident workgroup.
+    static constexpr int XPOSE_PITCH = 64 * 4 + 16, XPOSE_BYTES = 16 * XPOSE_PITCH;
+    static constexpr bool XPOSE = FN % 4 == 0 && OCC * (RING_BYTES + WAVES * XPOSE_BYTES) <= 160 * 1024;
+    static constexpr int LDS_BYTES = RING_BYTES + (XPOSE ? WAVES * XPOSE_BYTES : 0);
     // one DMA piece = one wave-wide 16-byte-per-lane load = 16 rows x 64 bytes
     static constexpr int A_PIECES = BM / 16 / WAVES, B_PIECES = BN / 16 / WAVES;
     static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile is a multiple of 16x16");
@@ -95,7 +102,7 @@ struct Tile16Cfg {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
     static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
     static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
-    static_assert(FM >= 2 && FM % 2 == 0 && FN >= 2 && FN % 2 == 0, "pipeline needs an even number (>= 2) of A fragments per wave; the epilogue pairs B fragments");
+    static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
     static_assert((12 * FN) % FM == 0, "B widening must split evenly over the sub-steps");
 };
 
@@ -296,73 +303,96 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     asm volatile("s_mov_b32 %0, 0xf0f0f0f0" : "=s"(amask));
 
     // ---- writing a finished tile ----
-    // A 16x16 block leaves the MFMA as 16 rows x 64 bytes per wave-wide store, and a CU
-    // pushes such half-line stores out more than three times slower than stores that
-    // cover whole 128-byte lines.  Two blocks that are neighbours along n hold, between
-    // them, 16 rows x 128 bytes; lanes r and r^8 (same 16-lane row of the wave) swap one
-    // block each, after which one store carries rows 0..7 and the next rows 8..15, both
-    // 128 bytes wide.
-    // this lane's place in the 16 x 32 area of two neighbouring blocks, after the swap
-    const int c_row = wm * Cfg::WM + (r & 7), c_col = wn * Cfg::WN + ((r >> 3) << 4) + g * 4;
-    // byte offset of that place from the tile's corner (32 bits are enough for the rows of one
-    // tile when N is below 2^21)
-    const uint32_t lane_c = ((uint32_t)c_row * (uint32_t)p.N + (uint32_t)c_col) * 4u;
+    // A 16x16 block leaves the MFMA with lane (r, g) holding row r, columns 4g..4g+3: a
+    // wave-wide 16-byte store of it touches 16 rows, and consecutive lanes sit in different
+    // rows.  The memory pipeline of a CU takes such stores more than three times slower
+    // than stores in which every 4 consecutive lanes cover 64 contiguous bytes (measured:
+    // 6.4 us against 2.1 us for the 256 KiB of one tile).  Where the LDS has room, four
+    // blocks that are neighbours along n (16 rows x 64 columns) therefore pass through a
+    // per-wave LDS area: written as they come, read back with 16 consecutive lanes per row
+    // (4 rows x 256 bytes per store).  The accumulators are only touched through asm
+    // statements: an ordinary read or write inside the loop makes the register allocator
+    // treat them as general values and copy them around.
     int c_item = blockIdx.x, c_kt = 0, c_m0, c_n0, c_kt0, c_KT;  // the item being contracted
     char *tile_c = nullptr;  // its corner in C (wave-uniform)
-    auto store_piece = [&](const int m, const int n, const v4i v) __attribute__((always_inline)) {
-        if (m >= p.M) return;
-        int32_t *crow = p.C + (size_t)m * p.N;
-        if (ksplit > 1) {
-            // every partial accumulator is a multiple of 256, so the shifted partials add
-            // up to the shifted total; integer atomics make the order irrelevant
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        } else if (vec_ok && n + 3 < p.N) {
-            *reinterpret_cast<v4i *>(crow + n) = v;
-        } else {
-            if (n < p.N) crow[n] = v.x;
-            if (n + 1 < p.N) crow[n + 1] = v.y;
-            if (n + 2 < p.N) crow[n + 2] = v.z;
-            if (n + 3 < p.N) crow[n + 3] = v.w;
-        }
-    };
     v4i zero4;
     asm volatile("v_mov_b32 %0, 0" : "=v"(zero4.x));  // (opaque, so the MFMA operand is a plain register tuple)
     zero4.y = zero4.z = zero4.w = zero4.x;
-    // The work for blocks (ib, j) and (ib, j+1), in four parts so that it can ride in four
-    // MFMA slots: read one block; read the other and clear both (the accumulators are only
-    // touched through asm statements: an ordinary read or write inside the loop makes the
-    // register allocator treat them as general values and copy them around); swap, drop
-    // the factor 256 and store rows 0..7; the same for rows 8..15.  `whole`: the tile lies
-    // inside the matrix and the stores need no guards (and no branches, which would cut
-    // the slot-by-slot schedule of a K-step apart).
-    v4i ex, ey;
-    auto write_part = [&](auto whole_, auto ib_, auto j_, auto q_) __attribute__((always_inline)) {
-        constexpr bool whole = decltype(whole_)::value;
-        constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value, q = decltype(q_)::value;
-        if constexpr (q == 0) {
+    // accumulator block -> registers, cleared behind the read, factor 256 dropped
+    auto take_block = [&](auto ib_, auto j_) __attribute__((always_inline)) -> v4i {
+        constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value;
+        v4i v;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ex[e] = acc_read(acc[ib][j][e]);
-        } else if constexpr (q == 1) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) ey[e] = acc_read(acc[ib][j + 1][e]);
-            mfma16_zero(acc[ib][j], zero4);
-            mfma16_zero(acc[ib][j + 1], zero4);
+        for (int e = 0; e < 4; ++e) v[e] = acc_read(acc[ib][j][e]);
+        mfma16_zero(acc[ib][j], zero4);
+        v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
+        return v;
+    };
+    // byte offsets of this lane from the tile's corner (32 bits are enough for the rows of one
+    // tile when N is below 2^21): as the MFMA leaves a block, and as the LDS area is read back
+    const uint32_t lane_blk = ((uint32_t)(wm * Cfg::WM + r) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + g * 4)) * 4u;
+    const uint32_t lane_row = ((uint32_t)(wm * Cfg::WM + (lane >> 4)) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + (lane & 15) * 4)) * 4u;
+    uint8_t *const xp = smem + Cfg::RING_BYTES + wave * Cfg::XPOSE_BYTES;
+    const int xp_wr = r * Cfg::XPOSE_PITCH + g * 16, xp_rd = (lane >> 4) * Cfg::XPOSE_PITCH + (lane & 15) * 16;
+    v4i xr[4];
+    // Whole tile, through the LDS: part t = 0..7 of blocks (ib, 4*grp .. 4*grp+3), one part per
+    // MFMA slot.  Parts 0..3 write one block each; the read-back of row quartet k and its
+    // store are two parts apart, so the store does not wait for the LDS.
+    auto write_group = [&](auto ib_, auto grp_, auto t_) __attribute__((always_inline)) {
+        constexpr int ib = decltype(ib_)::value, grp = decltype(grp_)::value, t = decltype(t_)::value;
+        auto read_back = [&](auto k_) __attribute__((always_inline)) {
+            constexpr int k = decltype(k_)::value;
+            xr[k] = *reinterpret_cast<const v4i *>(xp + xp_rd + 4 * k * Cfg::XPOSE_PITCH);
+        };
+        auto store_rows = [&](auto k_) __attribute__((always_inline)) {
+            constexpr int k = decltype(k_)::value;
+            char *const at = tile_c + ((size_t)(ib * 16 + 4 * k) * p.N + grp * 64) * 4;  // wave-uniform
+            *reinterpret_cast<v4i *>(at + lane_row) = xr[k];
+        };
+        if constexpr (t < 4)
+            *reinterpret_cast<v4i *>(xp + xp_wr + 64 * t) = take_block(ib_, std::integral_constant<int, 4 * grp + t>{});
+        if constexpr (t == 3) read_back(std::integral_constant<int, 0>{});
+        if constexpr (t == 4) read_back(std::integral_constant<int, 1>{});
+        if constexpr (t == 5) { read_back(std::integral_constant<int, 2>{}); store_rows(std::integral_constant<int, 0>{}); }
+        if constexpr (t == 6) { read_back(std::integral_constant<int, 3>{}); store_rows(std::integral_constant<int, 1>{}); }
+        if constexpr (t == 7) { store_rows(std::integral_constant<int, 2>{}); store_rows(std::integral_constant<int, 3>{}); }
+    };
+    // Whole tile, no room in the LDS: block (ib, j) stored as it is, in two parts.
+    auto write_block = [&](auto ib_, auto j_, auto t_) __attribute__((always_inline)) {
+        constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value, t = decltype(t_)::value;
+        if constexpr (t == 0) {
+            xr[0] = take_block(ib_, j_);
         } else {
-            // row_ror:8 pairs lane r with lane r^8; the bank mask picks the half that takes its
-            // partner's value (banks 2,3 = r >= 8; banks 0,1 = r < 8), the rest keep theirs
-            v4i v;
+            char *const at = tile_c + ((size_t)(ib * 16) * p.N + j * 16) * 4;  // wave-uniform
+            *reinterpret_cast<v4i *>(at + lane_blk) = xr[0];
+        }
+    };
+    // Slot s of 2*FN for the blocks of row ib of a whole tile
+    auto write_whole = [&](auto ib_, auto s_) __attribute__((always_inline)) {
+        constexpr int s = decltype(s_)::value;
+        if constexpr (Cfg::XPOSE) write_group(ib_, std::integral_constant<int, s / 8>{}, std::integral_constant<int, s % 8>{});
+        else write_block(ib_, std::integral_constant<int, s / 2>{}, std::integral_constant<int, s % 2>{});
+    };
+    // Any tile: guarded stores (ragged edges, odd N or unaligned C, K-split partial sums)
+    auto write_guarded = [&](auto ib_, auto j_) __attribute__((always_inline)) {
+        constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value;
+        const v4i v = take_block(ib_, j_);
+        const int m = (c_m0 + ib * 16) + (wm * Cfg::WM + r), n = (c_n0 + j * 16) + (wn * Cfg::WN + g * 4);
+        if (m < p.M) {
+            int32_t *crow = p.C + (size_t)m * p.N;
+            if (ksplit > 1) {
+                // every partial accumulator is a multiple of 256, so the shifted partials add
+                // up to the shifted total; integer atomics make the order irrelevant
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                v[e] = (q == 2 ? __builtin_amdgcn_update_dpp(ex[e], ey[e], 0x128, 0xF, 0xC, false)
-                               : __builtin_amdgcn_update_dpp(ey[e], ex[e], 0x128, 0xF, 0x3, false)) >> 8;
-            constexpr int row = ib * 16 + (q == 2 ? 0 : 8);
-            if constexpr (whole) {
-                char *const at = tile_c + ((size_t)row * p.N + j * 16) * 4;  // wave-uniform
-                *reinterpret_cast<v4i *>(at + lane_c) = v;
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else if (vec_ok && n + 3 < p.N) {
+                *reinterpret_cast<v4i *>(crow + n) = v;
             } else {
-                store_piece((c_m0 + row) + c_row, (c_n0 + j * 16) + c_col, v);
+                if (n < p.N) crow[n] = v.x;
+                if (n + 1 < p.N) crow[n + 1] = v.y;
+                if (n + 2 < p.N) crow[n + 2] = v.z;
+                if (n + 3 < p.N) crow[n + 3] = v.w;
             }
         }
     };
@@ -371,8 +401,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // bs), reads and widens the B fragments of the step in ring[1] with `bmask` (zero when
     // that step is an item's padding), and issues the cursor's loads into the last stage.
     // In the last step of a whole tile, row i-1 of the accumulator blocks is final once
-    // sub-step i begins: its write-out rides in the slots of sub-step i, two blocks per four
-    // slots, instead of stalling the matrix cores afterwards (row FM-1 is left to the caller).
+    // sub-step i begins: its write-out rides in the slots of sub-step i instead of stalling
+    // the matrix cores afterwards (row FM-1 is left to the caller).
     auto k_step = [&](const uint32_t bmask, auto bs_tag, auto last_tag) __attribute__((always_inline)) {
         constexpr int bs = decltype(bs_tag)::value;
         constexpr bool last = decltype(last_tag)::value;
@@ -412,9 +442,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     });
                 }
                 // -- write-out of the accumulator row finished one sub-step ago --
-                if constexpr (last && i >= 1)
-                    write_part(std::true_type{}, std::integral_constant<int, i - 1>{}, std::integral_constant<int, 2 * (s / 4)>{},
-                               std::integral_constant<int, s % 4>{});
+                if constexpr (last && i >= 1) write_whole(std::integral_constant<int, i - 1>{}, s_);
                 // -- DMA pieces of the step AHEAD of this one, one sub-step apart --
                 if constexpr (s == SLOTS - 1) {
                     static_for<0, NP>([&](auto q_) {
@@ -472,16 +500,21 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         static_for<(FN > 4 ? FN - 4 : 0), FN>([&](auto j_) {
             mfma16_settle(acc[FM - 1][decltype(j_)::value]);
         });
-        static_for<(whole ? FM - 1 : 0), FM>([&](auto ib_) {
-            static_for<0, FN / 2>([&](auto jp_) {
-                static_for<0, 4>([&](auto q_) {
-                    write_part(whole_, ib_, std::integral_constant<int, 2 * decltype(jp_)::value>{}, q_);
-                });
-                // one pair at a time: the widened fragments of the next step stay live
-                // across this code, so there are few registers to stage results in
+        if constexpr (whole) {
+            static_for<0, 2 * FN>([&](auto s_) {
+                write_whole(std::integral_constant<int, FM - 1>{}, s_);
                 __builtin_amdgcn_sched_barrier(0);
             });
-        });
+        } else {
+            static_for<0, FM>([&](auto ib_) {
+                static_for<0, FN>([&](auto j_) {
+                    write_guarded(ib_, j_);
+                    // one block at a time: the widened fragments of the next step stay live
+                    // across this code, so there are few registers to stage results in
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+            });
+        }
     };
     for (; c_item < nwhole; c_item += G) run_item(std::true_type{});
     for (; c_item < nitems; c_item += G) run_item(std::false_type{});
