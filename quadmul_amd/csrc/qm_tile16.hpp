@@ -54,6 +54,15 @@ __device__ __forceinline__ void mfma16_settle(v4i &acc)
     asm volatile("s_nop 15\n\ts_nop 15" : "+a"(acc));
 }
 
+// the 64-bit value (hi:lo) << 4, as one instruction (it issues faster than two
+// 32-bit shifts).
+__device__ __forceinline__ v2i shl4_pair(const int lo, const int hi)
+{
+    v2i in = {lo, hi}, out;
+    asm("v_lshlrev_b64 %0, 4, %1" : "=v"(out) : "v"(in));
+    return out;
+}
+
 // A use of `x` that generates no code: the value has to exist at this point of the program.
 __device__ __forceinline__ void keep_here(const v4i &x) { asm volatile("" ::"v"(x)); }
 
@@ -83,6 +92,7 @@ struct Tile16Cfg {
     static constexpr int WAVES = WGM * WGN, THREADS = 64 * WAVES;
     static constexpr int WM = BM / WGM, WN = BN / WGN;
     static constexpr int FM = WM / 16, FN = WN / 16;  // 16x16 accumulator blocks per wave
+    static constexpr int W_OPS = 10;                  // VALU instructions that widen one packed fragment
     static constexpr int PITCH = 64;                  // packed bytes per row per K-step
     static constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
@@ -103,7 +113,7 @@ struct Tile16Cfg {
     static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
     static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
     static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
-    static_assert((12 * FN) % FM == 0, "B widening must split evenly over the sub-steps");
+    static_assert((W_OPS * FN) % FM == 0, "B widening must split evenly over the sub-steps");
 };
 
 template <class Cfg>
@@ -288,12 +298,17 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
 #pragma unroll
     for (int t = 0; t < STAGES; ++t) ring[t] = t * STAGE;
 
-    // Widening op k (0..11) of a packed fragment: dword k/3; part 0: shift, 1: mask -> even
-    // nibbles, 2: mask -> odd nibbles.
-    auto widen_op = [&](auto k_, const v4i &pk, v4i &ev, v4i &od, const uint32_t mask) {
-        constexpr int k = decltype(k_)::value, d = k / 3, part = k % 3;
-        if constexpr (part == 0) ev[d] = (int)((uint32_t)pk[d] << 4);
-        else if constexpr (part == 1) ev[d] = (int)((uint32_t)ev[d] & mask);
+    // Widening op k (0..W-1) of a packed fragment, W = 10: for each half (dwords 2h, 2h+1) one
+    // 64-bit shift of the pair (the nibble that crosses into the upper dword is masked away
+    // with the rest), then a mask each for the even and the odd nibbles of both dwords.
+    auto widen_op = [&](auto k_, const v4i &pk, v4i &ev, v4i &od, const uint32_t mask) __attribute__((always_inline)) {
+        constexpr int k = decltype(k_)::value, h = k / 5, part = k % 5, d = 2 * h + (part - 1) / 2;
+        if constexpr (part == 0) {
+            const v2i t = shl4_pair(pk[2 * h], pk[2 * h + 1]);
+            ev[2 * h] = t.x;
+            ev[2 * h + 1] = t.y;
+        }
+        else if constexpr (part % 2 == 1) ev[d] = (int)((uint32_t)ev[d] & mask);
         else od[d] = (int)((uint32_t)pk[d] & mask);
     };
 
@@ -407,8 +422,9 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         constexpr int bs = decltype(bs_tag)::value;
         constexpr bool last = decltype(last_tag)::value;
         constexpr int SLOTS = 2 * FN;                // MFMAs per sub-step
-        constexpr int BSHARE = 12 * FN / FM;         // B widening ops per sub-step
-        constexpr int NOPS = 12 + BSHARE;            // VALU ops per sub-step, spread over slots 1..SLOTS-1
+        constexpr int W = Cfg::W_OPS;
+        constexpr int BSHARE = W * FN / FM;          // B widening ops per sub-step
+        constexpr int NOPS = W + BSHARE;             // VALU ops per sub-step, spread over slots 1..SLOTS-1
         static_for<0, FM>([&](auto i_) {
             constexpr int i = decltype(i_)::value;
             constexpr int pa = i & 1;
@@ -422,22 +438,22 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     //    sub-step, and the A fragment two sub-steps ahead --
                     static_for<0, FN>([&](auto j_) {
                         constexpr int j = decltype(j_)::value;
-                        if constexpr ((12 * j) / BSHARE == i) b_pk[j & 1] = read_b(ring[1], j);
+                        if constexpr ((W * j) / BSHARE == i) b_pk[j & 1] = read_b(ring[1], j);
                     });
                     constexpr int i2 = i + 2;
                     a_pk[pa] = read_a(i2 >= FM ? ring[1] : ring[0], i2 % FM);
                 } else {
                     // -- this slot's share of the widening work: ops [lo, hi) of the sub-step's
-                    //    list: 12 ops for the next A fragment, then BSHARE ops of the next B --
+                    //    list: W ops for the next A fragment, then BSHARE ops of the next B --
                     constexpr int lo = (s - 1) * NOPS / (SLOTS - 1), hi = s * NOPS / (SLOTS - 1);
                     static_for<lo, hi>([&](auto o_) {
                         constexpr int o = decltype(o_)::value;
-                        if constexpr (o < 12) {
+                        if constexpr (o < W) {
                             widen_op(std::integral_constant<int, o>{}, a_pk[pa ^ 1], a_ev[pa ^ 1], a_od[pa ^ 1], amask);
                         } else {
-                            constexpr int gop = i * BSHARE + (o - 12);  // index into the K-step's B op list
-                            constexpr int j = gop / 12;
-                            widen_op(std::integral_constant<int, gop % 12>{}, b_pk[j & 1], b_ev[bs ^ 1][j], b_od[bs ^ 1][j], bmask);
+                            constexpr int gop = i * BSHARE + (o - W);  // index into the K-step's B op list
+                            constexpr int j = gop / W;
+                            widen_op(std::integral_constant<int, gop % W>{}, b_pk[j & 1], b_ev[bs ^ 1][j], b_od[bs ^ 1][j], bmask);
                         }
                     });
                 }
