@@ -463,7 +463,10 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 if constexpr (s == SLOTS - 1) {
                     static_for<0, NP>([&](auto q_) {
                         constexpr int q = decltype(q_)::value;
-                        if constexpr (q * FM / NP == i) dma_piece(q, ring[STAGES - 1]);
+                        // (With a ring of three stages the loads issued in a step must have landed
+                        // at its end.  In a last step they all go out in sub-step 0, ahead of the
+                        // first store, so that "all but the stores" can be waited for.)
+                        if constexpr (last && AHEAD == 2 ? i == 0 : q * FM / NP == i) dma_piece(q, ring[STAGES - 1]);
                     });
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -482,9 +485,9 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         keep_here(a_pk[1]);
         // The step two ahead must have landed, and every wave must be done reading this
         // step's stage, before the roles rotate; the younger steps stay in flight.  The
-        // counter also counts the stores of a last step, which are younger than the loads
-        // that must have landed: they are allowed to stay in flight as well (the counter
-        // cannot express more than 63).
+        // counter counts loads and stores alike, in order of issue: the stores of a last
+        // step are all younger than the loads that must have landed, and are allowed to stay
+        // in flight as well (the counter cannot express more than 63).
         constexpr int pending = (AHEAD - 2) * NP + (last ? (FM - 1) * FN : 0);
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(pending > 63 ? 63 : pending) : "memory");
         const int t = ring[0];

@@ -285,6 +285,27 @@ def test_persistent_grid_many_items_per_workgroup(oracle_mod, shape):
     assert ran >= 4
 
 
+def test_many_rounds_repeated(oracle_mod):
+    """Many items per workgroup on every pipelined configuration, several times over: the
+    write-out of one tile overlaps the loads of the next, so a misplaced wait shows up as an
+    occasional wrong tile rather than every time (a three-stage ring once did exactly that)."""
+    m, n, k = 2048, 28672, 256
+    a, b = make_operands(m, n, k, SEED_BASE + 5100)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    want_d = fp32_matmul_on_gpu(a, b)
+    rows = np.arange(0, m, 127).astype(np.int32)
+    assert oracle_mod.compare(want_d.cpu().numpy()[rows], oracle_mod.gemm_i4_rows(ap.numpy(), bp.numpy(), rows)) == -1
+    for cfg, name in enumerate(qm.config_names()):
+        if not name.startswith("q"):
+            continue
+        for rep in range(6):
+            got_d = poisoned_c(m, n, DEV)
+            qm.gemm_cfg(a_d, b_d, got_d, m, n, k, cfg | ((1 + rep % 4) << 16))
+            torch.cuda.synchronize()
+            assert torch.equal(got_d, want_d), f"{name} repetition {rep}"
+
+
 @pytest.mark.parametrize("row", [(8, 8192, 8192, 8192), (9, 8000, 8000, 8064)], ids=lambda r: "x".join(map(str, r[1:])))
 def test_large_configs(oracle_mod, row):
     i, m, n, k = row
