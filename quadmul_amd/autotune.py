@@ -156,7 +156,7 @@ def emit_table(tuned: List[Dict], path: str) -> None:
     ]
     for t in tuned:
         b = t["best"]
-        lines.append(f"{{{t['m']}, {t['n']}, {t['k']}, \"{b['config']}\", {b['group_m']}, {b['ksplit']}}},  // {b['ms']*1e3:.1f} us, {b['tops']:.0f} TOPS")
+        lines.append(f"{{{t['m']}, {t['n']}, {t['k']}, \"{b['config']}\", {b['group_m']}, {b['ksplit']}, {b.get('spread', 0)}}},  // {b['ms']*1e3:.1f} us, {b['tops']:.0f} TOPS")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 

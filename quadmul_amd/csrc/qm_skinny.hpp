@@ -4,9 +4,15 @@
 // shapes outside its table are skipped (kernel.cu:340-385).  Here a workgroup
 // owns 16*FN rows of B (columns of C) and all of M (padded to 16*FM <= 64); its
 // NW waves split K between them in 128-nibble chunks, each wave streaming its
-// share of B straight from HBM into MFMA operand registers (16-byte loads, 64
-// contiguous bytes per row, no LDS on the way in), and the partial 16x16 blocks
-// are summed through LDS.  One launch, no workspace, no atomics, C overwritten.
+// share of B straight from HBM into registers, and the partial 16x16 blocks are
+// summed through LDS.  One launch, no workspace, no atomics, C overwritten.
+//
+// The MFMA wants lane r + 16 g to hold 16 bytes of row r (k-group g), which as a
+// load has consecutive lanes in different rows: the memory pipeline then handles
+// every lane's 16 bytes separately.  Lanes therefore load row lane/4, chunk lane%4
+// (4 consecutive lanes = 64 contiguous bytes) and a lane permutation through the
+// LDS crossbar (ds_bpermute, no LDS memory involved) puts the fragments into MFMA
+// order afterwards.
 #pragma once
 #include "qm_common.hpp"
 
@@ -36,11 +42,21 @@ gemm_skinny_kernel(const GemmArgs p)
 
     // Rows past the edge are clamped to a valid row; their products are dropped
     // by the store guards.
+    const int ld_row = lane >> 2, ld_ch = lane & 3;  // what this lane loads: row, 16-byte chunk
+    const int from_lane = (4 * r + g) * 4;           // where MFMA lane (r, g) finds its fragment (byte address of a lane)
     uint32_t b_off[FN], a_off[FM];
 #pragma unroll
-    for (int j = 0; j < FN; ++j) b_off[j] = (uint32_t)min(n0 + j * 16 + r, p.N - 1) * (uint32_t)Kb + g * 16;
+    for (int j = 0; j < FN; ++j) b_off[j] = (uint32_t)min(n0 + j * 16 + ld_row, p.N - 1) * (uint32_t)Kb + ld_ch * 16;
 #pragma unroll
-    for (int i = 0; i < FM; ++i) a_off[i] = (uint32_t)min(i * 16 + r, p.M - 1) * (uint32_t)Kb + g * 16;
+    for (int i = 0; i < FM; ++i) a_off[i] = (uint32_t)min(i * 16 + ld_row, p.M - 1) * (uint32_t)Kb + ld_ch * 16;
+    auto to_mfma_order = [&](const v4i q) -> v4i {
+        v4i o;
+        o.x = __builtin_amdgcn_ds_bpermute(from_lane, q.x);
+        o.y = __builtin_amdgcn_ds_bpermute(from_lane, q.y);
+        o.z = __builtin_amdgcn_ds_bpermute(from_lane, q.z);
+        o.w = __builtin_amdgcn_ds_bpermute(from_lane, q.w);
+        return o;
+    };
 
     v4i acc[FM][FN];
 #pragma unroll
@@ -55,7 +71,7 @@ gemm_skinny_kernel(const GemmArgs p)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int kofs = (c0 + u) * 64;
-            const bool ok = kofs + g * 16 < Kb;  // also false for c0+u >= nchunks
+            const bool ok = kofs + ld_ch * 16 < Kb;  // also false for c0+u >= nchunks
 #pragma unroll
             for (int j = 0; j < FN; ++j)
                 bq[u][j] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p.B + b_off[j] + kofs)) : v4i{0, 0, 0, 0};
@@ -67,11 +83,11 @@ gemm_skinny_kernel(const GemmArgs p)
         for (int u = 0; u < U; ++u) {
             v4i bev[FN], bod[FN];
 #pragma unroll
-            for (int j = 0; j < FN; ++j) x16_expand(bq[u][j], bev[j], bod[j]);
+            for (int j = 0; j < FN; ++j) x16_expand(to_mfma_order(bq[u][j]), bev[j], bod[j]);
 #pragma unroll
             for (int i = 0; i < FM; ++i) {
                 v4i aev, aod;
-                x16_expand(aq[u][i], aev, aod);
+                x16_expand(to_mfma_order(aq[u][i]), aev, aod);
 #pragma unroll
                 for (int j = 0; j < FN; ++j) acc[i][j] = mfma16(bev[j], aev, acc[i][j]);
 #pragma unroll
@@ -87,28 +103,18 @@ gemm_skinny_kernel(const GemmArgs p)
         for (int j = 0; j < FN; ++j) red[wave][i * FN + j][lane] = acc[i][j];
     __syncthreads();
 
-    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
-    for (int item = tid; item < FM * FN * 64; item += Cfg::THREADS) {
-        const int blk = item >> 6, l = item & 63;
-        v4i s = red[0][blk][l];
+    // One output element per thread and pass: element (m, n) of block blk sits in register
+    // n % 4 of lane m + 16 * (n / 4) of every wave's partial block; 16 consecutive threads
+    // write 64 contiguous bytes of a row of C.
+    const int32_t *red_i = reinterpret_cast<const int32_t *>(&red[0][0][0]);
+    for (int idx = tid; idx < FM * FN * 256; idx += Cfg::THREADS) {
+        const int blk = idx >> 8, ml = (idx >> 4) & 15, nl = idx & 15;
+        const int src = (blk * 64 + ml + 16 * (nl >> 2)) * 4 + (nl & 3);
+        int32_t s = 0;
 #pragma unroll
-        for (int w = 1; w < NW; ++w) {
-            const v4i t = red[w][blk][l];
-            s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
-        }
-        s.x >>= 8; s.y >>= 8; s.z >>= 8; s.w >>= 8;
-        const int m = (blk / FN) * 16 + (l & 15);
-        const int n = n0 + (blk % FN) * 16 + (l >> 4) * 4;
-        if (m >= p.M) continue;
-        int32_t *crow = p.C + (size_t)m * p.N;
-        if (vec_ok && n + 3 < p.N) {
-            *reinterpret_cast<v4i *>(crow + n) = s;
-        } else {
-            if (n < p.N) crow[n] = s.x;
-            if (n + 1 < p.N) crow[n + 1] = s.y;
-            if (n + 2 < p.N) crow[n + 2] = s.z;
-            if (n + 3 < p.N) crow[n + 3] = s.w;
-        }
+        for (int w = 0; w < NW; ++w) s += red_i[w * (FM * FN * 256) + src];
+        const int m = (blk / FN) * 16 + ml, n = n0 + (blk % FN) * 16 + nl;
+        if (m < p.M && n < p.N) p.C[(size_t)m * p.N + n] = s >> 8;
     }
 }
 
