@@ -102,15 +102,21 @@ def time_graph(fn, launches=200, replays=5):
     return best
 
 
+# Bytes moved per launch past the L2s, from rocprofv3 counter runs of `bench.py --workload W
+# --launches-only 20` (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads
+# for a 256 MiB device-to-device copy; summaries under profiles/).  Not measured live.
+MEASURED_TRAFFIC = {(4096, 4096, 4096): 118968897, (8192, 8192, 8192): 677105932, (16, 4096, 4096): 8961456}
+
+
 def roofline_of(m, n, k, bound, ms):
     ops = 2.0 * m * n * k
     if bound == "mfma":
         achieved = ops / ms / 1e9  # TOP/s
         return {"bound": "mfma", "achieved": round(achieved, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": None}
+                "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC.get((m, n, k))}
     achieved = algorithmic_bytes(m, n, k) / ms / 1e6  # GB/s
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None}
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get((m, n, k))}
 
 
 def run_workload(name, steps, warmup, check_rows=64):
