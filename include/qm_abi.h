@@ -35,7 +35,8 @@ extern "C" {
 #define QM_ERR_SHAPE         -2 /* m, n or k negative, k odd, or a size overflows int32     */
 #define QM_ERR_CONFIG        -3 /* cfg id unknown, or that config cannot run this shape     */
 #define QM_ERR_LAUNCH        -4 /* the HIP runtime refused the launch (see qm_last_hip_error) */
-#define QM_ERR_ALIGN         -5 /* C is not 4-byte aligned                                  */
+#define QM_ERR_ALIGN         -5 /* C is not 4-byte aligned (a 16-bit output: 2-byte)         */
+#define QM_ERR_DTYPE         -6 /* out_dtype is none of the QM_OUT_* values                 */
 
 #define QM_CFG_AUTO          -1 /* let the shape table / heuristic choose                   */
 
@@ -63,6 +64,28 @@ int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, int k, void 
  * grid whose workgroups each run several tiles back to back.
  */
 int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg);
+
+/*
+ * The GEMM with a dequantising epilogue fused in:
+ *   D[m][n] = round16( ((float)C[m][n] * row_scale[m]) * col_scale[n] )
+ * where C is the exact int32 product above, both multiplications are IEEE single
+ * precision in this order, and round16 rounds to nearest even into fp16 (QM_OUT_F16) or
+ * bfloat16 (QM_OUT_BF16).  D is [M, N] 16-bit, row-major; row_scale is [M], col_scale is
+ * [N], device pointers, either may be NULL for all ones.  No counterpart in the
+ * reference's code: its README.md:7 names fused epilogues as what the kernel is for
+ * (per-token activation scales x per-channel weight scales of an int4 linear layer);
+ * C (4 bytes per element, most of the traffic of the int32 form) is never written.
+ * Same calling rules as qm_gemm_i4.  The _cfg form takes a configuration as
+ * qm_gemm_i4_cfg does (no K split; QM_ERR_CONFIG when that configuration has no scaled
+ * output, see qm_config_has_scaled).
+ */
+#define QM_OUT_F16  1
+#define QM_OUT_BF16 2
+int qm_gemm_i4_scaled(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
+                      const float *col_scale, int out_dtype, void *stream);
+int qm_gemm_i4_scaled_cfg(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
+                          const float *col_scale, int out_dtype, void *stream, int cfg);
+int qm_config_has_scaled(int cfg); /* 1 / 0 */
 
 /* The configuration qm_gemm_i4 would pick for this shape (the table lookup the
  * reference does at kernel.cu:340-385, here with a heuristic fallback instead of

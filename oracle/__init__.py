@@ -11,8 +11,12 @@ from .qm_oracle import (  # noqa: F401
     gemm_i8,
     gemm_numpy,
     max_threads,
+    OUT_BF16,
+    OUT_F16,
     pack_i4,
     pack_numpy,
+    scale_round16,
+    scale_round16_numpy,
     unpack_i4,
     unpack_numpy,
 )

@@ -10,6 +10,14 @@
  *   qm_oracle_unpack_i4      <- unpack_int4_matrix   kernel.cu:387-408 (U4_TO_S4 at :387)
  *   qm_oracle_pack_i4        <- pack_b               test.py:6-15
  *   qm_oracle_compare        <- compare_results      kernel.cu:308-319
+ *   qm_oracle_scale_round16  <- nothing: the reference has no fused epilogue (its
+ *                               README.md:7 only names the idea).  The definition is this
+ *                               build's own: out = round16(((float)C * rs[m]) * cs[n]) in
+ *                               IEEE single precision, round to nearest even.  Pinned by
+ *                               exhaustive agreement of both conversions with numpy's
+ *                               float16 cast / a bit-level bfloat16 rule over sampled and
+ *                               boundary floats, by unit and power-of-two scales, and by
+ *                               torch's own float32 arithmetic (tests/test_oracle_pins.py).
  *
  * Parity status: the reference holds no golden vectors for this path (its only
  * test draws unseeded inputs, test.py:22-23, and accepts |diff|<=1,
@@ -132,6 +140,55 @@ QM_API long long qm_oracle_compare(const int32_t *got, const int32_t *want, long
     for (long long i = 0; i < size; ++i)
         if (got[i] != want[i]) return i;
     return -1;
+}
+
+/* fp32 -> fp16 bits, round to nearest even, IEEE (subnormals, overflow to inf, NaN kept). */
+static uint16_t f32_to_f16(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const uint32_t mag = x & 0x7FFFFFFFu;
+    if (mag > 0x7F800000u) return (uint16_t)(sign | 0x7E00u);                 /* NaN */
+    if (mag >= 0x47800000u) return (uint16_t)(sign | 0x7C00u);                /* >= 65536: inf (also inf) */
+    if (mag < 0x33000000u) return (uint16_t)sign;                             /* < 2^-25: rounds to zero */
+    uint32_t exp = mag >> 23, man = mag & 0x7FFFFFu;
+    uint32_t half, rest, halfway;
+    if (exp >= 113) {                                                         /* normal half */
+        half = ((exp - 112) << 10) | (man >> 13);
+        rest = man & 0x1FFFu;
+        halfway = 0x1000u;
+    } else {                                                                  /* subnormal half */
+        const uint32_t shift = 126 - exp;                                     /* 14..24 */
+        man |= 0x800000u;
+        half = man >> shift;
+        rest = man & ((1u << shift) - 1u);
+        halfway = 1u << (shift - 1);
+    }
+    if (rest > halfway || (rest == halfway && (half & 1u))) ++half;           /* carry into the exponent is right */
+    return (uint16_t)(sign | half);
+}
+
+static uint16_t f32_to_bf16(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    x += 0x7FFFu + ((x >> 16) & 1u);
+    return (uint16_t)(x >> 16);
+}
+
+/* out: 1 = fp16, 2 = bfloat16; rs / cs may be NULL (all ones) */
+QM_API int qm_oracle_scale_round16(const int32_t *C, const float *rs, const float *cs, uint16_t *D, int M, int N, int out)
+{
+    if (M < 0 || N < 0 || (out != 1 && out != 2)) return -1;
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            volatile float t = (float)C[(size_t)m * N + n] * (rs ? rs[m] : 1.0f);  /* two roundings, in this order */
+            const float y = t * (cs ? cs[n] : 1.0f);
+            D[(size_t)m * N + n] = out == 1 ? f32_to_f16(y) : f32_to_bf16(y);
+        }
+    return 0;
 }
 
 QM_API int qm_oracle_max_threads(void)

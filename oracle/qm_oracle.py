@@ -58,6 +58,8 @@ def _load():
     lib.qm_oracle_gemm_i4_rows.restype = ci
     lib.qm_oracle_compare.argtypes = [i32p, i32p, ctypes.c_longlong]
     lib.qm_oracle_compare.restype = ctypes.c_longlong
+    lib.qm_oracle_scale_round16.argtypes = [i32p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ci, ci, ci]
+    lib.qm_oracle_scale_round16.restype = ci
     lib.qm_oracle_max_threads.argtypes = []
     lib.qm_oracle_max_threads.restype = ci
     _lib = lib
@@ -153,6 +155,43 @@ def compare(got, want) -> int:
     if g.shape != w.shape:
         raise ValueError("shape mismatch")
     return int(_load().qm_oracle_compare(_ptr(g), _ptr(w), g.size))
+
+
+OUT_F16, OUT_BF16 = 1, 2
+
+
+def scale_round16(C, row_scale, col_scale, out: int) -> np.ndarray:
+    """uint16 bit patterns of round16(((float32)C * row_scale[m]) * col_scale[n]); ``out`` is
+    OUT_F16 or OUT_BF16; a scale of None stands for all ones.  (No counterpart in the reference.)"""
+    C = np.ascontiguousarray(C, dtype=np.int32)
+    M, N = C.shape
+    rs = None if row_scale is None else np.ascontiguousarray(row_scale, dtype=np.float32)
+    cs = None if col_scale is None else np.ascontiguousarray(col_scale, dtype=np.float32)
+    if (rs is not None and rs.shape != (M,)) or (cs is not None and cs.shape != (N,)):
+        raise ValueError("scale shapes")
+    D = np.empty((M, N), dtype=np.uint16)
+    rc = _load().qm_oracle_scale_round16(_ptr(C), None if rs is None else rs.ctypes.data, None if cs is None else cs.ctypes.data,
+                                         D.ctypes.data, M, N, out)
+    if rc < 0:
+        raise RuntimeError("qm_oracle_scale_round16 rejected its arguments")
+    return D
+
+
+def scale_round16_numpy(C, row_scale, col_scale, out: int) -> np.ndarray:
+    """The same in numpy: float32 products in the same order, numpy's own float16 cast, and
+    bfloat16 by the add-0x7FFF-plus-lsb rule on the bit pattern."""
+    y = np.asarray(C, dtype=np.int32).astype(np.float32)
+    if row_scale is not None:
+        y = (y * np.asarray(row_scale, dtype=np.float32)[:, None]).astype(np.float32)
+    if col_scale is not None:
+        y = (y * np.asarray(col_scale, dtype=np.float32)[None, :]).astype(np.float32)
+    if out == OUT_F16:
+        with np.errstate(over="ignore"):
+            return y.astype(np.float16).view(np.uint16)
+    u = y.view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    return np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), r)
 
 
 # ---------------------------------------------------------------- numpy restatement

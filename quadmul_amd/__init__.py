@@ -21,7 +21,8 @@ from typing import List, Optional
 import torch
 
 __all__ = [
-    "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "pack_int4", "unpack_int4",
+    "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "gemm_scaled", "pack_int4", "unpack_int4",
+    "config_has_scaled",
     "num_configs", "config_name", "config_names", "config_id", "select_config", "config_supports",
     "CFG_AUTO", "version",
 ]
@@ -33,7 +34,7 @@ _lib: Optional[ctypes.CDLL] = None
 CFG_AUTO = -1
 #: every symbol include/qm_abi.h declares
 ABI_SYMBOLS = (
-    "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_select_config", "qm_num_configs", "qm_config_name",
+    "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled", "qm_select_config", "qm_num_configs", "qm_config_name",
     "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version",
 )
 
@@ -61,6 +62,12 @@ def library() -> ctypes.CDLL:
     lib.qm_gemm_i4.restype = ci
     lib.qm_gemm_i4_cfg.argtypes = [vp, vp, vp, ci, ci, ci, vp, ci]
     lib.qm_gemm_i4_cfg.restype = ci
+    lib.qm_gemm_i4_scaled.argtypes = [vp, vp, vp, ci, ci, ci, vp, vp, ci, vp]
+    lib.qm_gemm_i4_scaled.restype = ci
+    lib.qm_gemm_i4_scaled_cfg.argtypes = [vp, vp, vp, ci, ci, ci, vp, vp, ci, vp, ci]
+    lib.qm_gemm_i4_scaled_cfg.restype = ci
+    lib.qm_config_has_scaled.argtypes = [ci]
+    lib.qm_config_has_scaled.restype = ci
     lib.qm_select_config.argtypes = [ci, ci, ci, ci]
     lib.qm_select_config.restype = ci
     lib.qm_num_configs.argtypes = []
@@ -101,7 +108,7 @@ def _is_byte(t: torch.Tensor) -> bool:
     return t.dtype in (torch.int8, torch.uint8)
 
 
-def _check_operands(a, b, c, m, n, k) -> None:
+def _check_operands(a, b, c, m, n, k, c_dtypes=(torch.int32,)) -> None:
     # The checks the reference left commented out (extension.cpp:11-15).
     if not (a.is_cuda and b.is_cuda and c.is_cuda):
         raise QuadmulError("gemm: a, b and c must be GPU tensors")
@@ -109,8 +116,8 @@ def _check_operands(a, b, c, m, n, k) -> None:
         raise QuadmulError("gemm: all tensors must be on the same device")
     if not (_is_byte(a) and _is_byte(b)):
         raise QuadmulError("gemm: a and b must be int8 or uint8 (packed int4)")
-    if c.dtype != torch.int32:
-        raise QuadmulError("gemm: c must be int32")
+    if c.dtype not in c_dtypes:
+        raise QuadmulError("gemm: c must be " + " or ".join(str(d).replace("torch.", "") for d in c_dtypes))
     if not (a.is_contiguous() and b.is_contiguous() and c.is_contiguous()):
         raise QuadmulError("gemm: all tensors must be contiguous")
     if m < 0 or n < 0 or k < 0 or k % 2:
@@ -129,6 +136,31 @@ def gemm_cfg(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, 
     with torch.cuda.device(a.device):
         st = library().qm_gemm_i4_cfg(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, _stream_ptr(a), cfg)
     _check(st, "qm_gemm_i4_cfg")
+
+
+def gemm_scaled(a: torch.Tensor, b: torch.Tensor, d: torch.Tensor, m: int, n: int, k: int,
+                row_scale: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None, cfg: int = CFG_AUTO) -> None:
+    """The GEMM with the dequantising epilogue fused in (no counterpart in the reference's
+    code; README.md:7 names the idea): ``d[m,n] = round(((float)c[m,n] * row_scale[m]) *
+    col_scale[n])`` with ``c`` the exact int32 product; ``d`` is float16 or bfloat16 and is
+    overwritten; the scales are float32 vectors on the same device, None = all ones."""
+    _check_operands(a, b, d, m, n, k, c_dtypes=(torch.float16, torch.bfloat16))
+    for s_, cnt, what in ((row_scale, m, "row_scale"), (col_scale, n, "col_scale")):
+        if s_ is None:
+            continue
+        if not (s_.is_cuda and s_.device == a.device and s_.dtype == torch.float32 and s_.is_contiguous() and s_.numel() == cnt):
+            raise QuadmulError(f"gemm_scaled: {what} must be a contiguous float32 vector of {cnt} elements on a's device")
+    out = 1 if d.dtype == torch.float16 else 2
+    with torch.cuda.device(a.device):
+        st = library().qm_gemm_i4_scaled_cfg(a.data_ptr(), b.data_ptr(), d.data_ptr(), m, n, k,
+                                             None if row_scale is None else row_scale.data_ptr(),
+                                             None if col_scale is None else col_scale.data_ptr(), out, _stream_ptr(a), cfg)
+    _check(st, "qm_gemm_i4_scaled")
+
+
+def config_has_scaled(cfg: int) -> bool:
+    """Whether configuration ``cfg`` exists with the scaled 16-bit float output."""
+    return bool(library().qm_config_has_scaled(cfg))
 
 
 def gemm(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int) -> None:

@@ -29,13 +29,18 @@ bool is_byte(const torch::Tensor &t) { return t.scalar_type() == torch::kInt8 ||
 
 void *stream_of(const torch::Tensor &t) { return static_cast<void *>(c10::hip::getCurrentHIPStream(t.get_device()).stream()); }
 
-void check_operands(const torch::Tensor &a, const torch::Tensor &b, const torch::Tensor &c, int64_t m, int64_t n, int64_t k)
+void check_operands(const torch::Tensor &a, const torch::Tensor &b, const torch::Tensor &c, int64_t m, int64_t n, int64_t k,
+                    bool scaled = false)
 {
     TORCH_CHECK(a.is_cuda() && b.is_cuda() && c.is_cuda(), "quadmul.gemm: a, b and c must be GPU tensors");
     TORCH_CHECK(a.device() == b.device() && a.device() == c.device(), "quadmul.gemm: all tensors must be on the same device");
     // pack_b yields int8 (test.py:14); the reference only ever looks at data_ptr().
     TORCH_CHECK(is_byte(a) && is_byte(b), "quadmul.gemm: a and b must be int8 or uint8 (packed int4)");
-    TORCH_CHECK(c.scalar_type() == torch::kInt32, "quadmul.gemm: c must be int32");
+    if (scaled) {
+        TORCH_CHECK(c.scalar_type() == torch::kFloat16 || c.scalar_type() == torch::kBFloat16, "quadmul.gemm_scaled: d must be float16 or bfloat16");
+    } else {
+        TORCH_CHECK(c.scalar_type() == torch::kInt32, "quadmul.gemm: c must be int32");
+    }
     TORCH_CHECK(a.is_contiguous() && b.is_contiguous() && c.is_contiguous(), "quadmul.gemm: all tensors must be contiguous");
     TORCH_CHECK(m >= 0 && n >= 0 && k >= 0 && k % 2 == 0, "quadmul.gemm: m, n, k must be >= 0 and k even");
     TORCH_CHECK(m <= INT32_MAX && n <= INT32_MAX && k <= INT32_MAX, "quadmul.gemm: m, n, k must fit in int32");
@@ -49,6 +54,30 @@ void gemm(torch::Tensor a, torch::Tensor b, torch::Tensor c, int64_t m, int64_t 
     check_operands(a, b, c, m, n, k);
     c10::OptionalDeviceGuard guard(a.device());
     check_status(qm_gemm_i4(a.data_ptr(), b.data_ptr(), c.data_ptr(), (int)m, (int)n, (int)k, stream_of(a)), "quadmul.gemm");
+}
+
+// The GEMM with the dequantising epilogue fused in (no counterpart in the reference's code;
+// its README.md:7 names the idea): d = round(((float)c * row_scale[m]) * col_scale[n]), d
+// float16 or bfloat16, the scales float32 vectors on a's device (an undefined tensor = ones).
+void check_scale(const c10::optional<torch::Tensor> &s, const torch::Tensor &a, int64_t count, const char *what)
+{
+    if (!s.has_value()) return;
+    TORCH_CHECK(s->is_cuda() && s->device() == a.device() && s->scalar_type() == torch::kFloat32 && s->is_contiguous() && s->numel() == count,
+                "quadmul.gemm_scaled: ", what, " must be a contiguous float32 vector of ", count, " elements on a's device");
+}
+
+void gemm_scaled(torch::Tensor a, torch::Tensor b, torch::Tensor d, int64_t m, int64_t n, int64_t k,
+                 c10::optional<torch::Tensor> row_scale, c10::optional<torch::Tensor> col_scale)
+{
+    check_operands(a, b, d, m, n, k, true);
+    check_scale(row_scale, a, m, "row_scale");
+    check_scale(col_scale, a, n, "col_scale");
+    c10::OptionalDeviceGuard guard(a.device());
+    const int out = d.scalar_type() == torch::kFloat16 ? QM_OUT_F16 : QM_OUT_BF16;
+    check_status(qm_gemm_i4_scaled(a.data_ptr(), b.data_ptr(), d.data_ptr(), (int)m, (int)n, (int)k,
+                                   row_scale.has_value() ? row_scale->data_ptr<float>() : nullptr,
+                                   col_scale.has_value() ? col_scale->data_ptr<float>() : nullptr, out, stream_of(a)),
+                 "quadmul.gemm_scaled");
 }
 
 void gemm_cfg(torch::Tensor a, torch::Tensor b, torch::Tensor c, int64_t m, int64_t n, int64_t k, int64_t cfg)
@@ -87,16 +116,37 @@ torch::Tensor unpack(torch::Tensor packed)
 // cannot see through.  c is written in place; nothing is returned.
 void gemm_meta(const torch::Tensor &, const torch::Tensor &, torch::Tensor &, int64_t, int64_t, int64_t) {}
 void gemm_op(const torch::Tensor &a, const torch::Tensor &b, torch::Tensor &c, int64_t m, int64_t n, int64_t k) { gemm(a, b, c, m, n, k); }
+void gemm_scaled_meta(const torch::Tensor &, const torch::Tensor &, torch::Tensor &, int64_t, int64_t, int64_t,
+                      const c10::optional<torch::Tensor> &, const c10::optional<torch::Tensor> &) {}
+void gemm_scaled_op(const torch::Tensor &a, const torch::Tensor &b, torch::Tensor &d, int64_t m, int64_t n, int64_t k,
+                    const c10::optional<torch::Tensor> &row_scale, const c10::optional<torch::Tensor> &col_scale)
+{
+    gemm_scaled(a, b, d, m, n, k, row_scale, col_scale);
+}
 
 }  // namespace
 
-TORCH_LIBRARY(quadmul, m) { m.def("gemm(Tensor a, Tensor b, Tensor(c!) c, int m, int n, int k) -> ()"); }
-TORCH_LIBRARY_IMPL(quadmul, CUDA, m) { m.impl("gemm", &gemm_op); }
-TORCH_LIBRARY_IMPL(quadmul, Meta, m) { m.impl("gemm", &gemm_meta); }
+TORCH_LIBRARY(quadmul, m)
+{
+    m.def("gemm(Tensor a, Tensor b, Tensor(c!) c, int m, int n, int k) -> ()");
+    m.def("gemm_scaled(Tensor a, Tensor b, Tensor(d!) d, int m, int n, int k, Tensor? row_scale, Tensor? col_scale) -> ()");
+}
+TORCH_LIBRARY_IMPL(quadmul, CUDA, m)
+{
+    m.impl("gemm", &gemm_op);
+    m.impl("gemm_scaled", &gemm_scaled_op);
+}
+TORCH_LIBRARY_IMPL(quadmul, Meta, m)
+{
+    m.impl("gemm", &gemm_meta);
+    m.impl("gemm_scaled", &gemm_scaled_meta);
+}
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     m.def("gemm", &gemm, "Int4xInt4 Matrix Multiplication Kernel", py::arg("a"), py::arg("b"), py::arg("c"), py::arg("m"), py::arg("n"), py::arg("k"));
+    m.def("gemm_scaled", &gemm_scaled, "Int4xInt4 GEMM with per-row and per-column fp32 scales, fp16 / bf16 output", py::arg("a"), py::arg("b"),
+          py::arg("d"), py::arg("m"), py::arg("n"), py::arg("k"), py::arg("row_scale") = py::none(), py::arg("col_scale") = py::none());
     m.def("gemm_cfg", &gemm_cfg, "gemm with an explicit kernel configuration id (autotuning)");
     m.def("pack", &pack, "Pack a [rows, K] int8 tensor of int4 values into [rows, K/2] bytes on the GPU");
     m.def("unpack", &unpack, "Unpack [rows, K/2] bytes into a [rows, K] int8 tensor on the GPU");

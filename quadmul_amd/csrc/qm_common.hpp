@@ -8,12 +8,55 @@ namespace qm {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 
+// Output forms: the exact int32 product, or the product scaled per row and per column in
+// fp32 and rounded to a 16-bit float (the "dequantise on the way out" use the reference's
+// README.md:7 has in mind; no code of the reference does it).
+enum OutKind { OUT_I32 = 0, OUT_F16 = 1, OUT_BF16 = 2 };
+
 struct GemmArgs {
     const uint8_t *A;  // [M, K/2] packed s4
     const uint8_t *B;  // [N, K/2] packed s4
-    int32_t *C;        // [M, N]
+    int32_t *C;        // [M, N] int32; or [M, N] 16-bit floats when `out` says so
     int M, N, K;
+    // scaled output only: D[m][n] = round16(((float)C[m][n] * row_scale[m]) * col_scale[n]),
+    // a null pointer standing for all ones
+    const float *row_scale = nullptr;  // [M]
+    const float *col_scale = nullptr;  // [N]
+    int out = OUT_I32;
 };
+
+__device__ __forceinline__ float scale_at(const float *s, int i, int n) { return (s != nullptr && i < n) ? s[i] : 1.0f; }
+
+// fp32 -> 16-bit float, round to nearest even (NaN stays NaN).  Contraction is switched
+// off in these helpers: fused, the compiler turns "multiply, then round to fp16" into one
+// instruction with a single rounding, which is not the value defined above.
+template <int OUT>
+__device__ __forceinline__ uint16_t round16(float x)
+{
+#pragma clang fp contract(off)
+    if constexpr (OUT == OUT_F16) {
+        // (the empty asm hides where x came from: instruction selection otherwise merges a
+        // preceding fp32 multiply and this conversion into v_fma_mixlo_f16, which rounds the
+        // exact product once, straight to fp16 -- not the twice-rounded value defined above)
+        asm("" : "+v"(x));
+        const _Float16 h = (_Float16)x;
+        return __builtin_bit_cast(uint16_t, h);
+    } else {
+        // (both candidates computed and one selected: no per-lane branch in the callers' code)
+        const uint32_t u = __builtin_bit_cast(uint32_t, x);
+        const uint32_t rounded = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16, quiet = (u >> 16) | 0x0040u;
+        return (uint16_t)(((u & 0x7FFFFFFFu) > 0x7F800000u) ? quiet : rounded);
+    }
+}
+__device__ __forceinline__ uint16_t round16(float x, int out) { return out == OUT_F16 ? round16<OUT_F16>(x) : round16<OUT_BF16>(x); }
+
+// the scaled value of one element, in the one order of operations everything here uses
+__device__ __forceinline__ float scaled(int c, float rs, float cs)
+{
+#pragma clang fp contract(off)
+    const float t = (float)c * rs;
+    return t * cs;
+}
 
 // gfx950 has no int4 MFMA, so nibbles are widened to int8 -- but scaled by 16,
 // which needs no per-byte sign fix-up.  For a dword w holding nibbles k0..k7

@@ -46,7 +46,12 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(const GemmArgs p, con
         }
         __syncthreads();
     }
-    if (m0 + ty < p.M && n0 + tx < p.N) p.C[(size_t)(m0 + ty) * p.N + n0 + tx] = sum;
+    const int m = m0 + ty, n = n0 + tx;
+    if (m < p.M && n < p.N) {
+        const size_t at = (size_t)m * p.N + n;
+        if (p.out == OUT_I32) p.C[at] = sum;
+        else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(sum, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
+    }
 }
 
 static hipError_t launch_generic(const GemmArgs &p, hipStream_t stream, int)
@@ -61,6 +66,11 @@ static hipError_t launch_generic(const GemmArgs &p, hipStream_t stream, int)
 // Zero fill (k == 0) and pack / unpack, flat over the whole array: K is even so
 // a byte never straddles two rows.
 // --------------------------------------------------------------------------
+__global__ void fill_zero16_kernel(uint16_t *dst, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = 0;
+}
+
 __global__ void fill_zero_kernel(int32_t *dst, size_t n)
 {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = 0;
@@ -172,6 +182,26 @@ static const ConfigDesc g_configs[] = {
 };
 static constexpr int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
+// Pipelined configurations that also exist with the scaled 16-bit float output
+static const struct { const char *name; LaunchFn launch; } g_scaled_tile16[] = {
+#define QM_TILE16S(tu, BM, BN, WGM, WGN, ST, OCC) \
+    {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_s" QM_STR(ST) "o" QM_STR(OCC), &QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC)},
+#include "qm_configs.inc"
+};
+
+// The launcher of configuration cfg for the scaled output, or null: the generic and the
+// skinny kernels take the output form at run time, the pipelined ones as separate kernels,
+// the plain tile kernels not at all.
+static LaunchFn scaled_launcher(int cfg)
+{
+    const ConfigDesc &c = g_configs[cfg];
+    if (c.kind == KIND_GENERIC || c.kind == KIND_SKINNY) return c.launch;
+    if (c.kind == KIND_TILE16)
+        for (const auto &e : g_scaled_tile16)
+            if (std::strcmp(e.name, c.name) == 0) return e.launch;
+    return nullptr;
+}
+
 static int find_config(const char *name)
 {
     for (int i = 0; i < g_num_configs; ++i)
@@ -271,6 +301,32 @@ static Choice select_config(int m, int n, int k, int ptr_align)
     return heuristic(m, n, k, ptr_align);
 }
 
+// The scaled output has fewer kernels to choose from: the table's choice when that
+// configuration has the output form, else the best pipelined one that has it, else what the
+// heuristic says for skinny shapes, else the generic kernel.
+static Choice select_scaled(int m, int n, int k, int ptr_align)
+{
+    const Choice ch = select_config(m, n, k, ptr_align);
+    if (ch.ksplit <= 1 && scaled_launcher(ch.cfg)) return ch;
+    if (fast_path_ok(m, n, k, ptr_align) && k % 128 == 0) {
+        int best = -1;
+        double best_cost = 1e300;
+        for (const auto &e : g_scaled_tile16) {
+            const int id = find_config(e.name);
+            if (id < 0) continue;
+            const ConfigDesc &d = g_configs[id];
+            const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
+            const double eff = d.bm * d.bn >= 256 * 256 ? 1.0 : (d.bm * d.bn >= 256 * 128 ? 0.82 : 0.66);
+            const double cost = (double)((tiles + 255) / 256) * d.bm * d.bn / eff;
+            if (cost < best_cost) { best_cost = cost; best = id; }
+        }
+        if (best >= 0) return {best, 4, 1};
+    }
+    const Choice h = heuristic(m, n, k, ptr_align);
+    if (h.ksplit <= 1 && scaled_launcher(h.cfg)) return h;
+    return {0, 1, 1};
+}
+
 static thread_local int g_last_hip_error = 0;
 
 static int ptr_alignment(const void *a, const void *b)
@@ -339,6 +395,57 @@ QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n
     return e == hipSuccess ? QM_OK : fail_launch(e);
 }
 
+QM_EXPORT int qm_gemm_i4_scaled_cfg(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
+                                    const float *col_scale, int out_dtype, void *stream, int cfg)
+{
+    if (out_dtype != QM_OUT_F16 && out_dtype != QM_OUT_BF16) return QM_ERR_DTYPE;
+    if (m < 0 || n < 0 || k < 0 || (k & 1)) return QM_ERR_SHAPE;
+    if (m == 0 || n == 0) return QM_OK;
+    if (!D) return QM_ERR_NULL;
+    if ((uintptr_t)D & 1) return QM_ERR_ALIGN;
+    if (k > 0 && (!A || !B)) return QM_ERR_NULL;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (k == 0) {
+        const size_t cnt = (size_t)m * (size_t)n;
+        fill_zero16_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<uint16_t *>(D), cnt);
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? QM_OK : fail_launch(e);
+    }
+    const int align = ptr_alignment(A, B);
+    Choice ch;
+    if (cfg == QM_CFG_AUTO) {
+        ch = select_scaled(m, n, k, align);
+    } else {
+        ch.cfg = cfg & 0xFFFF;
+        ch.group_m = (cfg >> 16) & 0xFF;
+        ch.ksplit = 1;
+        ch.spread = (cfg >> 30) & 1;
+        if (ch.group_m == 0) ch.group_m = 4;
+        if (((cfg >> 24) & 0x3F) > 1) return QM_ERR_CONFIG;  // partial sums cannot meet in a rounded output
+        if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
+    }
+    const LaunchFn launch = scaled_launcher(ch.cfg);
+    if (!launch) return QM_ERR_CONFIG;
+    GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(D), m, n, k};
+    p.row_scale = row_scale;
+    p.col_scale = col_scale;
+    p.out = out_dtype == QM_OUT_F16 ? OUT_F16 : OUT_BF16;
+    const hipError_t e = launch(p, s, ch.group_m | (1 << 8) | (ch.spread << 16));
+    return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
+QM_EXPORT int qm_gemm_i4_scaled(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
+                                const float *col_scale, int out_dtype, void *stream)
+{
+    return qm_gemm_i4_scaled_cfg(A, B, D, m, n, k, row_scale, col_scale, out_dtype, stream, QM_CFG_AUTO);
+}
+
+QM_EXPORT int qm_config_has_scaled(int cfg)
+{
+    cfg &= 0xFFFF;
+    return (cfg >= 0 && cfg < g_num_configs && scaled_launcher(cfg)) ? 1 : 0;
+}
+
 QM_EXPORT int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, int k, void *stream)
 {
     return qm_gemm_i4_cfg(A, B, C, m, n, k, stream, QM_CFG_AUTO);
@@ -402,7 +509,8 @@ QM_EXPORT const char *qm_status_string(int status)
     case QM_ERR_SHAPE: return "bad shape (m, n, k must be >= 0 and k even)";
     case QM_ERR_CONFIG: return "unknown kernel configuration, or it cannot run this shape";
     case QM_ERR_LAUNCH: return "HIP launch failed";
-    case QM_ERR_ALIGN: return "C must be 4-byte aligned";
+    case QM_ERR_ALIGN: return "C must be 4-byte aligned (a 16-bit output 2-byte aligned)";
+    case QM_ERR_DTYPE: return "unknown output type";
     default: return "unknown status";
     }
 }

@@ -114,7 +114,11 @@ gemm_skinny_kernel(const GemmArgs p)
 #pragma unroll
         for (int w = 0; w < NW; ++w) s += red_i[w * (FM * FN * 256) + src];
         const int m = (blk / FN) * 16 + ml, n = n0 + (blk % FN) * 16 + nl;
-        if (m < p.M && n < p.N) p.C[(size_t)m * p.N + n] = s >> 8;
+        if (m < p.M && n < p.N) {
+            const size_t at = (size_t)m * p.N + n;
+            if (p.out == OUT_I32) p.C[at] = s >> 8;
+            else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s >> 8, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
+        }
     }
 }
 

@@ -66,6 +66,8 @@ __device__ __forceinline__ v2i shl4_pair(const int lo, const int hi)
 // A use of `x` that generates no code: the value has to exist at this point of the program.
 __device__ __forceinline__ void keep_here(const v4i &x) { asm volatile("" ::"v"(x)); }
 
+__device__ __forceinline__ void keep_here_f(const float &x) { asm volatile("" ::"v"(x)); }
+
 // One accumulator register -> ordinary register.  Inside the loop the accumulators are
 // touched by asm statements only: an ordinary read there makes the register allocator
 // treat them as general values, and it starts moving and spilling them.
@@ -73,6 +75,16 @@ __device__ __forceinline__ int acc_read(const int acc_elem)
 {
     int dst;
     asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(dst) : "a"(acc_elem));
+    return dst;
+}
+// The same with two wait states in front, for the first read of a block: the destination
+// registers may be the data of a 16-byte store or ds_write issued just before, which the
+// hardware is still reading; the compiler pads that hazard for its own instructions but
+// does not look inside asm statements.
+__device__ __forceinline__ int acc_read_first(const int acc_elem)
+{
+    int dst;
+    asm volatile("s_nop 1\n\tv_accvgpr_read_b32 %0, %1" : "=v"(dst) : "a"(acc_elem));
     return dst;
 }
 
@@ -116,13 +128,14 @@ struct Tile16Cfg {
     static_assert((W_OPS * FN) % FM == 0, "B widening must split evenly over the sub-steps");
 };
 
-template <class Cfg>
+template <class Cfg, int OUT = OUT_I32>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::OCC * Cfg::THREADS / 256)
 gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const int group_m, const int ksplit)
 {
     constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, FM = Cfg::FM, FN = Cfg::FN;
     constexpr int PITCH = Cfg::PITCH, STAGE = Cfg::STAGE_BYTES, WAVES = Cfg::WAVES;
     constexpr int A_PIECES = Cfg::A_PIECES, B_PIECES = Cfg::B_PIECES, NP = A_PIECES + B_PIECES;
+    constexpr int ESZ = OUT == OUT_I32 ? 4 : 2;  // bytes per element of the output
 
     // (Every lambda below is marked always_inline: the state they share -- accumulators,
     // ring, load cursor -- lives in registers only as long as nothing is outlined.)
@@ -159,7 +172,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // column and bottom row of tiles; or all items, when nwhole is 0), written out by the
     // guarded code after the last K-step.  A workgroup's items ascend, so it runs its whole
     // tiles first and then the rest: two loops one after the other.
-    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & 15) == 0;
+    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & (4 * ESZ - 1)) == 0;  // 4 elements per store
     const bool plain_c = vec_ok && ksplit == 1 && p.N < (1 << 21);
     const int full_m = p.M / BM, full_n = p.N / BN;
     const int nwhole = __builtin_amdgcn_readfirstlane(plain_c ? full_m * full_n : 0);
@@ -330,6 +343,11 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // treat them as general values and copy them around.
     int c_item = blockIdx.x, c_kt = 0, c_m0, c_n0, c_kt0, c_KT;  // the item being contracted
     char *tile_c = nullptr;  // its corner in C (wave-uniform)
+    // scaled output: this lane's scales for the item, as the MFMA leaves a block (row r of
+    // every block row, columns 4g..4g+3 of every block column)
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    float rs_reg[OUT != OUT_I32 ? FM : 1];
+    v4f cs_reg[OUT != OUT_I32 ? FN : 1];
     v4i zero4;
     asm volatile("v_mov_b32 %0, 0" : "=v"(zero4.x));  // (opaque, so the MFMA operand is a plain register tuple)
     zero4.y = zero4.z = zero4.w = zero4.x;
@@ -338,15 +356,30 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value;
         v4i v;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc_read(acc[ib][j][e]);
+        for (int e = 0; e < 4; ++e) v[e] = e == 0 ? acc_read_first(acc[ib][j][e]) : acc_read(acc[ib][j][e]);
         mfma16_zero(acc[ib][j], zero4);
         v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
+        if constexpr (OUT != OUT_I32) {
+            // scaled output: from here on the four registers hold fp32 bit patterns
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = __builtin_bit_cast(int, scaled(v[e], rs_reg[ib], cs_reg[j][e]));
+        }
         return v;
+    };
+    // four fp32 bit patterns -> four 16-bit floats in two registers
+    auto pack16 = [&](const v4i v) __attribute__((always_inline)) -> v2i {
+        uint32_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int bits = v[e];  // (by value: a bit cast applied to the vector element itself reads element 0)
+            h[e] = round16<OUT == OUT_I32 ? OUT_F16 : OUT>(__builtin_bit_cast(float, bits));
+        }
+        return v2i{(int)(h[0] | (h[1] << 16)), (int)(h[2] | (h[3] << 16))};
     };
     // byte offsets of this lane from the tile's corner (32 bits are enough for the rows of one
     // tile when N is below 2^21): as the MFMA leaves a block, and as the LDS area is read back
-    const uint32_t lane_blk = ((uint32_t)(wm * Cfg::WM + r) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + g * 4)) * 4u;
-    const uint32_t lane_row = ((uint32_t)(wm * Cfg::WM + (lane >> 4)) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + (lane & 15) * 4)) * 4u;
+    const uint32_t lane_blk = ((uint32_t)(wm * Cfg::WM + r) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + g * 4)) * (uint32_t)ESZ;
+    const uint32_t lane_row = ((uint32_t)(wm * Cfg::WM + (lane >> 4)) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + (lane & 15) * 4)) * (uint32_t)ESZ;
     uint8_t *const xp = smem + Cfg::RING_BYTES + wave * Cfg::XPOSE_BYTES;
     const int xp_wr = r * Cfg::XPOSE_PITCH + g * 16, xp_rd = (lane >> 4) * Cfg::XPOSE_PITCH + (lane & 15) * 16;
     v4i xr[4];
@@ -361,8 +394,9 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         };
         auto store_rows = [&](auto k_) __attribute__((always_inline)) {
             constexpr int k = decltype(k_)::value;
-            char *const at = tile_c + ((size_t)(ib * 16 + 4 * k) * p.N + grp * 64) * 4;  // wave-uniform
-            *reinterpret_cast<v4i *>(at + lane_row) = xr[k];
+            char *const at = tile_c + ((size_t)(ib * 16 + 4 * k) * p.N + grp * 64) * ESZ;  // wave-uniform
+            if constexpr (OUT == OUT_I32) *reinterpret_cast<v4i *>(at + lane_row) = xr[k];
+            else *reinterpret_cast<v2i *>(at + lane_row) = pack16(xr[k]);
         };
         if constexpr (t < 4)
             *reinterpret_cast<v4i *>(xp + xp_wr + 64 * t) = take_block(ib_, std::integral_constant<int, 4 * grp + t>{});
@@ -378,8 +412,9 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         if constexpr (t == 0) {
             xr[0] = take_block(ib_, j_);
         } else {
-            char *const at = tile_c + ((size_t)(ib * 16) * p.N + j * 16) * 4;  // wave-uniform
-            *reinterpret_cast<v4i *>(at + lane_blk) = xr[0];
+            char *const at = tile_c + ((size_t)(ib * 16) * p.N + j * 16) * ESZ;  // wave-uniform
+            if constexpr (OUT == OUT_I32) *reinterpret_cast<v4i *>(at + lane_blk) = xr[0];
+            else *reinterpret_cast<v2i *>(at + lane_blk) = pack16(xr[0]);
         }
     };
     // Slot s of 2*FN for the blocks of row ib of a whole tile
@@ -393,7 +428,20 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value;
         const v4i v = take_block(ib_, j_);
         const int m = (c_m0 + ib * 16) + (wm * Cfg::WM + r), n = (c_n0 + j * 16) + (wn * Cfg::WN + g * 4);
-        if (m < p.M) {
+        if constexpr (OUT != OUT_I32) {
+            if (m < p.M) {
+                uint16_t *drow = reinterpret_cast<uint16_t *>(p.C) + (size_t)m * p.N;
+                const v2i o = pack16(v);
+                if (vec_ok && n + 3 < p.N) {
+                    *reinterpret_cast<v2i *>(drow + n) = o;
+                } else {
+                    if (n < p.N) drow[n] = (uint16_t)o.x;
+                    if (n + 1 < p.N) drow[n + 1] = (uint16_t)((uint32_t)o.x >> 16);
+                    if (n + 2 < p.N) drow[n + 2] = (uint16_t)o.y;
+                    if (n + 3 < p.N) drow[n + 3] = (uint16_t)((uint32_t)o.y >> 16);
+                }
+            }
+        } else if (m < p.M) {
             int32_t *crow = p.C + (size_t)m * p.N;
             if (ksplit > 1) {
                 // every partial accumulator is a multiple of 256, so the shifted partials add
@@ -502,6 +550,23 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     auto run_item = [&](auto whole_) __attribute__((always_inline)) {
         constexpr bool whole = decltype(whole_)::value;
         locate(c_item, c_m0, c_n0, c_kt0, c_KT);
+        if constexpr (OUT != OUT_I32) {
+            // The item's scales, loaded now and waited for now: the compiler cannot see the
+            // asm loads of the ring in the memory counter, so a wait it placed at the first
+            // use -- inside the last K-step -- would drain the whole ring there.
+#pragma unroll
+            for (int ib = 0; ib < FM; ++ib) rs_reg[ib] = scale_at(p.row_scale, c_m0 + wm * Cfg::WM + ib * 16 + r, p.M);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) cs_reg[j][e] = scale_at(p.col_scale, c_n0 + wn * Cfg::WN + j * 16 + g * 4 + e, p.N);
+#pragma unroll
+            for (int ib = 0; ib < FM; ++ib) keep_here_f(rs_reg[ib]);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) keep_here_f(cs_reg[j][e]);
+        }
         for (c_kt = 0; c_kt + 2 < c_KT; c_kt += 2) {
             k_step(amask, std::integral_constant<int, 0>{}, std::false_type{});
             k_step(amask, std::integral_constant<int, 1>{}, std::false_type{});
@@ -510,7 +575,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         // compiler would hoist the whole widening of B out of the MFMA slots into a branch)
         uint32_t bmask = c_kt + 1 < c_KT ? amask : 0u;
         asm volatile("" : "+s"(bmask));
-        tile_c = reinterpret_cast<char *>(p.C + ((size_t)c_m0 * p.N + c_n0));
+        tile_c = reinterpret_cast<char *>(p.C) + ((size_t)c_m0 * p.N + c_n0) * ESZ;
         k_step(bmask, std::integral_constant<int, 0>{}, std::false_type{});
         k_step(amask, std::integral_constant<int, 1>{}, std::integral_constant<bool, whole>{});
         // Let the last MFMAs retire before their accumulators are read (the compiler does not

@@ -30,7 +30,8 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 // zero-filled C when it is above 1) and, in bit 16, "one work item per workgroup".  By
 // default the grid is persistent: as many workgroups as the device holds at once, each
 // running several (K split, tile) items back to back.
-template <class Cfg, class Kernel>
+// (OUT is a template parameter so that every kernel gets launcher statics of its own.)
+template <class Cfg, int OUT, class Kernel>
 static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
 {
     static bool lds_ok[QM_MAX_DEVICES] = {};
@@ -85,8 +86,18 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
     hipError_t QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &p, hipStream_t s, int gm) \
     {                                                                                            \
         using Cfg = Tile16Cfg<BM, BN, WGM, WGN, ST, OCC>;                                        \
-        return launch_tiled_persistent<Cfg>(&gemm_tile16_kernel<Cfg>, p, s, gm);                   \
-    }                                                                                   \
+        return launch_tiled_persistent<Cfg, OUT_I32>(&gemm_tile16_kernel<Cfg, OUT_I32>, p, s, gm);  \
+    }                                                                                            \
+    }
+// the same configuration with the scaled 16-bit float outputs
+#define QM_TILE16S_DEF(BM, BN, WGM, WGN, ST, OCC)                                                 \
+    namespace qm {                                                                                \
+    hipError_t QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &p, hipStream_t s, int gm) \
+    {                                                                                             \
+        using Cfg = Tile16Cfg<BM, BN, WGM, WGN, ST, OCC>;                                         \
+        if (p.out == OUT_F16) return launch_tiled_persistent<Cfg, OUT_F16>(&gemm_tile16_kernel<Cfg, OUT_F16>, p, s, gm); \
+        return launch_tiled_persistent<Cfg, OUT_BF16>(&gemm_tile16_kernel<Cfg, OUT_BF16>, p, s, gm); \
+    }                                                                                             \
     }
 
 // An entry of qm_configs.inc is compiled here only when its unit number equals QM_TU:
@@ -99,6 +110,10 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK_5(...)
 #define QM_PICK_6(...)
 #define QM_PICK_7(...)
+#define QM_PICK_8(...)
+#define QM_PICK_9(...)
+#define QM_PICK_10(...)
+#define QM_PICK_11(...)
 #define QM_PICK16_0(...)
 #define QM_PICK16_1(...)
 #define QM_PICK16_2(...)
@@ -107,50 +122,111 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16_5(...)
 #define QM_PICK16_6(...)
 #define QM_PICK16_7(...)
+#define QM_PICK16_8(...)
+#define QM_PICK16_9(...)
+#define QM_PICK16_10(...)
+#define QM_PICK16_11(...)
+#define QM_PICK16S_0(...)
+#define QM_PICK16S_1(...)
+#define QM_PICK16S_2(...)
+#define QM_PICK16S_3(...)
+#define QM_PICK16S_4(...)
+#define QM_PICK16S_5(...)
+#define QM_PICK16S_6(...)
+#define QM_PICK16S_7(...)
+#define QM_PICK16S_8(...)
+#define QM_PICK16S_9(...)
+#define QM_PICK16S_10(...)
+#define QM_PICK16S_11(...)
 #if QM_TU == 0
 #undef QM_PICK_0
 #define QM_PICK_0(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_0
 #define QM_PICK16_0(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_0
+#define QM_PICK16S_0(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 1
 #undef QM_PICK_1
 #define QM_PICK_1(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_1
 #define QM_PICK16_1(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_1
+#define QM_PICK16S_1(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 2
 #undef QM_PICK_2
 #define QM_PICK_2(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_2
 #define QM_PICK16_2(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_2
+#define QM_PICK16S_2(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 3
 #undef QM_PICK_3
 #define QM_PICK_3(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_3
 #define QM_PICK16_3(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_3
+#define QM_PICK16S_3(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 4
 #undef QM_PICK_4
 #define QM_PICK_4(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_4
 #define QM_PICK16_4(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_4
+#define QM_PICK16S_4(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 5
 #undef QM_PICK_5
 #define QM_PICK_5(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_5
 #define QM_PICK16_5(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_5
+#define QM_PICK16S_5(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 6
 #undef QM_PICK_6
 #define QM_PICK_6(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_6
 #define QM_PICK16_6(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_6
+#define QM_PICK16S_6(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 7
 #undef QM_PICK_7
 #define QM_PICK_7(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_7
 #define QM_PICK16_7(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_7
+#define QM_PICK16S_7(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 8
+#undef QM_PICK_8
+#define QM_PICK_8(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_8
+#define QM_PICK16_8(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_8
+#define QM_PICK16S_8(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 9
+#undef QM_PICK_9
+#define QM_PICK_9(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_9
+#define QM_PICK16_9(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_9
+#define QM_PICK16S_9(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 10
+#undef QM_PICK_10
+#define QM_PICK_10(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_10
+#define QM_PICK16_10(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_10
+#define QM_PICK16S_10(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 11
+#undef QM_PICK_11
+#define QM_PICK_11(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_11
+#define QM_PICK16_11(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_11
+#define QM_PICK16S_11(...) QM_TILE16S_DEF(__VA_ARGS__)
 #else
 #error "QM_TU out of range"
 #endif
 
 #define QM_TILE(tu, ...) QM_PICK_##tu(__VA_ARGS__)
 #define QM_TILE16(tu, ...) QM_PICK16_##tu(__VA_ARGS__)
+#define QM_TILE16S(tu, ...) QM_PICK16S_##tu(__VA_ARGS__)
 #include "qm_configs.inc"

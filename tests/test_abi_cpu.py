@@ -34,6 +34,7 @@ def test_extension_module_imports_and_mirrors_reference_entry_point():
     assert callable(quadmul.gemm)
     assert "Int4xInt4 Matrix Multiplication Kernel" in quadmul.gemm.__doc__  # extension.cpp:28
     assert quadmul.num_configs() == qm.num_configs()
+    assert callable(quadmul.gemm_scaled)
 
 
 def test_dispatcher_op_is_registered_with_a_mutation_schema():
@@ -44,6 +45,9 @@ def test_dispatcher_op_is_registered_with_a_mutation_schema():
     assert [a.name for a in schema.arguments] == ["a", "b", "c", "m", "n", "k"]
     assert schema.arguments[2].alias_info is not None and schema.arguments[2].alias_info.is_write
     assert len(schema.returns) == 0
+    scaled = torch.ops.quadmul.gemm_scaled.default._schema
+    assert [a.name for a in scaled.arguments] == ["a", "b", "d", "m", "n", "k", "row_scale", "col_scale"]
+    assert scaled.arguments[2].alias_info is not None and scaled.arguments[2].alias_info.is_write
     # the Meta kernel lets a tracer run the op without data
     a = torch.empty((4, 16), dtype=torch.int8, device="meta")
     c = torch.empty((4, 4), dtype=torch.int32, device="meta")

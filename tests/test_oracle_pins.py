@@ -162,3 +162,61 @@ def test_golden_fixture_matches_oracle(oracle_mod):
     assert (oracle_mod.gemm_i4(z["a_packed"], z["b_packed"], threads=1) == z["c"]).all()
     assert (oracle_mod.gemm_numpy(z["a_packed"], z["b_packed"]) == z["c"]).all()
     assert (oracle_mod.unpack_i4(z["a_packed"]) == z["a"]).all()
+
+
+# ---------------------------------------------------------------- scaled 16-bit output
+# (no counterpart in the reference: pinned by exhaustive / boundary behaviour of the two
+# conversions and by two other statements of the same float32 arithmetic)
+def _f32(bits):
+    return np.asarray(bits, dtype=np.uint32).view(np.float32)
+
+
+def test_round16_conversions_against_numpy_and_bit_rules(oracle_mod):
+    rng = np.random.default_rng(7)
+    # every float16 value and the floats halfway between neighbours, just below and just above
+    h = np.arange(0, 0x7C00, dtype=np.uint16)
+    lo, hi = h.view(np.float16).astype(np.float32), (h + 1).astype(np.uint16).view(np.float16).astype(np.float32)
+    mid = ((lo.astype(np.float64) + hi.astype(np.float64)) / 2).astype(np.float32)  # exact: one more bit
+    cand = np.concatenate([lo, mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(np.inf)),
+                           _f32(rng.integers(0, 0x7F800000, 200000)), _f32([0x7F800000, 0x7FC00000, 0x477FE000, 0x477FF000, 0x33000000, 0x33000001, 0x32FFFFFF])])
+    cand = np.concatenate([cand, -cand]).astype(np.float32)
+    ones_r, ones_c = np.ones(1, np.float32), None
+    # feed the floats through the scale path: C = 1, row scale = the float itself
+    C = np.ones((cand.size, 1), dtype=np.int32)
+    got16 = oracle_mod.scale_round16(C, cand, None, oracle_mod.OUT_F16)[:, 0]
+    with np.errstate(over="ignore"):
+        want16 = cand.astype(np.float16).view(np.uint16)
+    nan = np.isnan(cand)
+    assert (got16[~nan] == want16[~nan]).all()
+    assert ((got16[nan] & 0x7C00) == 0x7C00).all() and ((got16[nan] & 0x03FF) != 0).all()
+    gotb = oracle_mod.scale_round16(C, cand, None, oracle_mod.OUT_BF16)[:, 0]
+    # bfloat16: nearest-even on the upper 16 bits, checked by value: |x - bf| <= half an ulp, ties to even
+    ok = ~nan & np.isfinite(cand)
+    bf = (gotb.astype(np.uint32) << 16).view(np.float32)
+    x64, b64 = cand[ok].astype(np.float64), bf[ok].astype(np.float64)
+    fin = np.isfinite(b64)
+    ulp = np.maximum(np.abs(b64[fin]), 2.0 ** -126) * 2.0 ** -7
+    assert (np.abs(x64[fin] - b64[fin]) <= ulp / 2 * 1.0000001 + 0).all()
+    exact = (cand.view(np.uint32) & 0xFFFF) == 0
+    assert (gotb[exact & ~nan] == (cand.view(np.uint32)[exact & ~nan] >> 16)).all()
+    tie = (cand.view(np.uint32) & 0xFFFF) == 0x8000
+    assert ((gotb[tie & ok] & 1) == 0).all()
+
+
+def test_scaled_output_against_numpy_and_torch(oracle_mod):
+    rng = np.random.default_rng(8)
+    C = rng.integers(-64 * 11008, 64 * 11008, size=(37, 129), dtype=np.int32)
+    C[0, :4] = [0, 1, -1, 2 ** 24 + 1]  # (the last one is not exactly representable in float32)
+    rs = rng.uniform(1e-4, 2.0, 37).astype(np.float32)
+    cs = rng.uniform(1e-5, 0.5, 129).astype(np.float32)
+    for out, tdt in ((oracle_mod.OUT_F16, torch.float16), (oracle_mod.OUT_BF16, torch.bfloat16)):
+        got = oracle_mod.scale_round16(C, rs, cs, out)
+        assert (got == oracle_mod.scale_round16_numpy(C, rs, cs, out)).all()
+        y = (torch.from_numpy(C).to(torch.float32) * torch.from_numpy(rs)[:, None]) * torch.from_numpy(cs)[None, :]
+        assert (got == y.to(tdt).view(torch.int16).numpy().view(np.uint16)).all()
+        # unit and power-of-two scales commute with the rounding of small integers
+        small = rng.integers(-2048, 2049, size=(5, 7), dtype=np.int32)
+        one = oracle_mod.scale_round16(small, None, None, out)
+        assert (one == torch.from_numpy(small).to(tdt).view(torch.int16).numpy().view(np.uint16)).all()
+        two = oracle_mod.scale_round16(small, np.full(5, 0.25, np.float32), np.full(7, 8.0, np.float32), out)
+        assert (two == (torch.from_numpy(small).to(torch.float32) * 2).to(tdt).view(torch.int16).numpy().view(np.uint16)).all()
