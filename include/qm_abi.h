@@ -108,6 +108,21 @@ int         qm_config_supports(int cfg, int m, int n, int k, int ptr_align); /* 
 int qm_pack_i4(const void *src_i8, void *dst_packed, int rows, int k, void *stream);
 int qm_unpack_i4(const void *src_packed, void *dst_i8, int rows, int k, void *stream);
 
+/*
+ * Quantise and pack in one pass: the step before the GEMM when the activations of an int4
+ * linear layer arrive as floats.  Per row r of x ([rows, k], row-major, fp16 / bf16 / fp32):
+ *   amax = max_j |x[r][j]|,  scales[r] = amax / 7,
+ *   q[j] = clamp(rint(x[r][j] * (7 / amax)), -7, 7)        (all zero when amax == 0)
+ * in IEEE single precision with round-half-to-even, packed as qm_pack_i4 packs (the
+ * packing half is pack_b, test.py:6-15; the reference has no quantiser: its test draws
+ * int4 values directly, test.py:22-23).  scales is [rows] float32 and is what
+ * qm_gemm_i4_scaled takes as row_scale.  x must be finite.  Each row is read from HBM once.
+ */
+#define QM_IN_F16  1
+#define QM_IN_BF16 2
+#define QM_IN_F32  3
+int qm_quantize_pack_i4(const void *x, int in_dtype, void *dst_packed, float *scales, int rows, int k, void *stream);
+
 /* Diagnostics. */
 const char *qm_status_string(int status);
 int         qm_last_hip_error(void);      /* hipError_t of the last failed launch on this thread */

@@ -15,6 +15,8 @@ from .qm_oracle import (  # noqa: F401
     OUT_F16,
     pack_i4,
     pack_numpy,
+    quantize_pack,
+    quantize_pack_numpy,
     scale_round16,
     scale_round16_numpy,
     unpack_i4,

@@ -10,6 +10,13 @@
  *   qm_oracle_unpack_i4      <- unpack_int4_matrix   kernel.cu:387-408 (U4_TO_S4 at :387)
  *   qm_oracle_pack_i4        <- pack_b               test.py:6-15
  *   qm_oracle_compare        <- compare_results      kernel.cu:308-319
+ *   qm_oracle_quantize_pack  <- nothing in the reference (activations arrive already
+ *                               quantised, test.py:22-23); its packing half is pack_b
+ *                               (test.py:6-15).  Definition, this build's own: per row,
+ *                               amax = max|x|, scale = amax / 7, q = clamp(rint(x * (7 / amax)),
+ *                               -7, 7) in IEEE single precision (q = 0 when amax = 0).  Pinned
+ *                               by exactly representable cases, by a numpy restatement and
+ *                               by round trips (tests/test_oracle_pins.py).
  *   qm_oracle_scale_round16  <- nothing: the reference has no fused epilogue (its
  *                               README.md:7 only names the idea).  The definition is this
  *                               build's own: out = round16(((float)C * rs[m]) * cs[n]) in
@@ -188,6 +195,34 @@ QM_API int qm_oracle_scale_round16(const int32_t *C, const float *rs, const floa
             const float y = t * (cs ? cs[n] : 1.0f);
             D[(size_t)m * N + n] = out == 1 ? f32_to_f16(y) : f32_to_bf16(y);
         }
+    return 0;
+}
+
+/* x: [rows, k] fp32 (callers widen fp16 / bf16 exactly); packed: [rows, k/2]; scales: [rows] */
+QM_API int qm_oracle_quantize_pack(const float *x, uint8_t *packed, float *scales, int rows, int k)
+{
+    if (rows < 0 || k < 0 || (k & 1)) return -1;
+    for (int r = 0; r < rows; ++r) {
+        const float *xr = x + (size_t)r * k;
+        float amax = 0.0f;
+        for (int j = 0; j < k; ++j) {
+            const float a = xr[j] < 0 ? -xr[j] : xr[j];
+            if (a > amax) amax = a;
+        }
+        const float inv = amax > 0.0f ? 7.0f / amax : 0.0f;
+        scales[r] = amax / 7.0f;
+        for (int j = 0; j < k; j += 2) {
+            int q[2];
+            for (int t = 0; t < 2; ++t) {
+                volatile float y = xr[j + t] * inv;
+                float rr = __builtin_rintf(y);           /* round half to even (default rounding mode) */
+                if (rr > 7.0f) rr = 7.0f;
+                if (rr < -7.0f) rr = -7.0f;
+                q[t] = (int)rr;
+            }
+            packed[(size_t)r * (k / 2) + j / 2] = (uint8_t)((q[0] & 0xF) | ((q[1] & 0xF) << 4));  /* test.py:8,14 */
+        }
+    }
     return 0;
 }
 

@@ -60,6 +60,8 @@ def _load():
     lib.qm_oracle_compare.restype = ctypes.c_longlong
     lib.qm_oracle_scale_round16.argtypes = [i32p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ci, ci, ci]
     lib.qm_oracle_scale_round16.restype = ci
+    lib.qm_oracle_quantize_pack.argtypes = [ctypes.c_void_p, u8p, ctypes.c_void_p, ci, ci]
+    lib.qm_oracle_quantize_pack.restype = ci
     lib.qm_oracle_max_threads.argtypes = []
     lib.qm_oracle_max_threads.restype = ci
     _lib = lib
@@ -158,6 +160,31 @@ def compare(got, want) -> int:
 
 
 OUT_F16, OUT_BF16 = 1, 2
+
+
+def quantize_pack(x):
+    """Per-row symmetric int4 quantisation fused with pack_b's packing (no counterpart in the
+    reference).  ``x``: [rows, k] float32 (widen fp16 / bf16 first: exact).  Returns (packed
+    uint8 [rows, k/2], scales float32 [rows]) with scale = amax / 7 and
+    q = clamp(rint(x * (7 / amax)), -7, 7)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rows, k = x.shape
+    packed = np.empty((rows, k // 2), dtype=np.uint8)
+    scales = np.empty(rows, dtype=np.float32)
+    rc = _load().qm_oracle_quantize_pack(x.ctypes.data, _ptr(packed), scales.ctypes.data, rows, k)
+    if rc < 0:
+        raise RuntimeError("qm_oracle_quantize_pack rejected its arguments")
+    return packed, scales
+
+
+def quantize_pack_numpy(x):
+    """The same in numpy (float32 throughout, np.rint = round half to even)."""
+    x = np.asarray(x, dtype=np.float32)
+    amax = np.abs(x).max(axis=1) if x.shape[1] else np.zeros(x.shape[0], np.float32)
+    with np.errstate(divide="ignore"):
+        inv = np.where(amax > 0, np.float32(7.0) / amax, np.float32(0)).astype(np.float32)
+    q = np.clip(np.rint((x * inv[:, None]).astype(np.float32)), -7, 7).astype(np.int8)
+    return pack_numpy(q), (amax / np.float32(7.0)).astype(np.float32)
 
 
 def scale_round16(C, row_scale, col_scale, out: int) -> np.ndarray:

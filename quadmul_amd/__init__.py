@@ -22,7 +22,7 @@ import torch
 
 __all__ = [
     "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "gemm_scaled", "pack_int4", "unpack_int4",
-    "config_has_scaled",
+    "config_has_scaled", "quantize_pack",
     "num_configs", "config_name", "config_names", "config_id", "select_config", "config_supports",
     "CFG_AUTO", "version",
 ]
@@ -34,7 +34,7 @@ _lib: Optional[ctypes.CDLL] = None
 CFG_AUTO = -1
 #: every symbol include/qm_abi.h declares
 ABI_SYMBOLS = (
-    "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled", "qm_select_config", "qm_num_configs", "qm_config_name",
+    "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled", "qm_quantize_pack_i4", "qm_select_config", "qm_num_configs", "qm_config_name",
     "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version",
 )
 
@@ -68,6 +68,8 @@ def library() -> ctypes.CDLL:
     lib.qm_gemm_i4_scaled_cfg.restype = ci
     lib.qm_config_has_scaled.argtypes = [ci]
     lib.qm_config_has_scaled.restype = ci
+    lib.qm_quantize_pack_i4.argtypes = [vp, ci, vp, vp, ci, ci, vp]
+    lib.qm_quantize_pack_i4.restype = ci
     lib.qm_select_config.argtypes = [ci, ci, ci, ci]
     lib.qm_select_config.restype = ci
     lib.qm_num_configs.argtypes = []
@@ -156,6 +158,27 @@ def gemm_scaled(a: torch.Tensor, b: torch.Tensor, d: torch.Tensor, m: int, n: in
                                              None if row_scale is None else row_scale.data_ptr(),
                                              None if col_scale is None else col_scale.data_ptr(), out, _stream_ptr(a), cfg)
     _check(st, "qm_gemm_i4_scaled")
+
+
+def quantize_pack(x: torch.Tensor):
+    """Per-row symmetric int4 quantisation fused with the packing, on the GPU (no counterpart
+    in the reference; the packing half is pack_b, test.py:6-15).  ``x``: [rows, k] float16,
+    bfloat16 or float32, contiguous.  Returns ``(packed int8 [rows, k/2], scales float32
+    [rows])`` with ``scales = amax / 7`` -- the ``row_scale`` of ``gemm_scaled``."""
+    if not (x.is_cuda and x.dim() == 2 and x.is_contiguous()):
+        raise QuadmulError("quantize_pack: x must be a contiguous 2-d GPU tensor")
+    kinds = {torch.float16: 1, torch.bfloat16: 2, torch.float32: 3}
+    if x.dtype not in kinds:
+        raise QuadmulError("quantize_pack: x must be float16, bfloat16 or float32")
+    rows, k = x.shape
+    if k % 2:
+        raise QuadmulError("quantize_pack: k must be even")
+    packed = torch.empty((rows, k // 2), dtype=torch.int8, device=x.device)
+    scales = torch.empty((rows,), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        st = library().qm_quantize_pack_i4(x.data_ptr(), kinds[x.dtype], packed.data_ptr(), scales.data_ptr(), rows, k, _stream_ptr(x))
+    _check(st, "qm_quantize_pack_i4")
+    return packed, scales
 
 
 def config_has_scaled(cfg: int) -> bool:

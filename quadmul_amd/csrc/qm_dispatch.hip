@@ -130,6 +130,157 @@ __global__ void unpack_i4_byte_kernel(const uint8_t *__restrict__ src, int8_t *_
     }
 }
 
+// --------------------------------------------------------------------------
+// Per-row symmetric quantisation to int4 fused with the packing: one workgroup per row,
+// the row held in registers between the two passes over it (maximum, then quantise), so
+// HBM is read once.  x is fp16, bf16 or fp32; 8 elements (4 packed bytes) per thread-chunk.
+// --------------------------------------------------------------------------
+template <int IN> struct QuantIn;
+template <> struct QuantIn<QM_IN_F16> {
+    static constexpr int BYTES = 2;
+    static __device__ __forceinline__ float widen(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+};
+template <> struct QuantIn<QM_IN_BF16> {
+    static constexpr int BYTES = 2;
+    static __device__ __forceinline__ float widen(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
+};
+template <> struct QuantIn<QM_IN_F32> {
+    static constexpr int BYTES = 4;
+};
+
+template <int IN>
+__device__ __forceinline__ void load8(const uint8_t *src, float (&v)[8])
+{
+    if constexpr (IN == QM_IN_F32) {
+        const v4i lo = *reinterpret_cast<const v4i *>(src), hi = *reinterpret_cast<const v4i *>(src + 16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int a = lo[e], b = hi[e];
+            v[e] = __builtin_bit_cast(float, a);
+            v[4 + e] = __builtin_bit_cast(float, b);
+        }
+    } else {
+        const v4i w = *reinterpret_cast<const v4i *>(src);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t d = (uint32_t)w[e];
+            v[2 * e] = QuantIn<IN>::widen((uint16_t)(d & 0xFFFFu));
+            v[2 * e + 1] = QuantIn<IN>::widen((uint16_t)(d >> 16));
+        }
+    }
+}
+
+__device__ __forceinline__ uint32_t quant8(const float (&v)[8], float inv)
+{
+#pragma clang fp contract(off)
+    uint32_t out = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float r = __builtin_rintf(v[e] * inv);  // round half to even
+        r = fminf(fmaxf(r, -7.0f), 7.0f);
+        out |= ((uint32_t)(int)r & 0xFu) << (4 * e);  // element e -> nibble e: low nibble = even k (test.py:8,14)
+    }
+    return out;
+}
+
+// workgroup-wide maximum of non-negative floats
+__device__ __forceinline__ float block_max(float x, float *lds)
+{
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) x = fmaxf(x, __shfl_xor(x, off));
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) lds[wave] = x;
+    __syncthreads();
+    float m = lds[0];
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) m = fmaxf(m, lds[w]);
+    __syncthreads();
+    return m;
+}
+
+// NC: chunks of 8 elements a thread keeps in registers (k <= 2048 * NC); NC == 0: any k that is
+// a multiple of 8, the row read twice (the second time out of the L2)
+template <int IN, int NC>
+__global__ void __launch_bounds__(256) quantize_pack_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ dst, float *__restrict__ scales, int k)
+{
+    __shared__ float red[4];
+    const int row = blockIdx.x, tid = threadIdx.x, nchunks = k >> 3;
+    const uint8_t *xr = x + (size_t)row * k * QuantIn<IN>::BYTES;
+    uint32_t *out = reinterpret_cast<uint32_t *>(dst + (size_t)row * (k >> 1));
+    float amax = 0.0f;
+    if constexpr (NC > 0) {
+        float v[NC][8];
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+            const int c = tid + i * 256;
+            if (c < nchunks) {
+                load8<IN>(xr + (size_t)c * 8 * QuantIn<IN>::BYTES, v[i]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[i][e]));
+            }
+        }
+        amax = block_max(amax, red);
+        const float inv = amax > 0.0f ? 7.0f / amax : 0.0f;
+        if (tid == 0) scales[row] = amax / 7.0f;
+#pragma unroll
+        for (int i = 0; i < NC; ++i) {
+            const int c = tid + i * 256;
+            if (c < nchunks) out[c] = quant8(v[i], inv);
+        }
+    } else {
+        float v[8];
+        for (int c = tid; c < nchunks; c += 256) {
+            load8<IN>(xr + (size_t)c * 8 * QuantIn<IN>::BYTES, v);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
+        }
+        amax = block_max(amax, red);
+        const float inv = amax > 0.0f ? 7.0f / amax : 0.0f;
+        if (tid == 0) scales[row] = amax / 7.0f;
+        for (int c = tid; c < nchunks; c += 256) {
+            load8<IN>(xr + (size_t)c * 8 * QuantIn<IN>::BYTES, v);
+            out[c] = quant8(v, inv);
+        }
+    }
+}
+
+// any even k, any alignment: one pair of elements per thread and pass
+template <int IN>
+__global__ void __launch_bounds__(256) quantize_pack_scalar_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ dst, float *__restrict__ scales, int k)
+{
+#pragma clang fp contract(off)
+    __shared__ float red[4];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    auto at = [&](int j) -> float {
+        if constexpr (IN == QM_IN_F32) {
+            return reinterpret_cast<const float *>(x)[(size_t)row * k + j];
+        } else {
+            return QuantIn<IN>::widen(reinterpret_cast<const uint16_t *>(x)[(size_t)row * k + j]);
+        }
+    };
+    float amax = 0.0f;
+    for (int j = tid; j < k; j += 256) amax = fmaxf(amax, fabsf(at(j)));
+    amax = block_max(amax, red);
+    const float inv = amax > 0.0f ? 7.0f / amax : 0.0f;
+    if (tid == 0) scales[row] = amax / 7.0f;
+    for (int j = 2 * tid; j < k; j += 512) {
+        const float r0 = fminf(fmaxf(__builtin_rintf(at(j) * inv), -7.0f), 7.0f), r1 = fminf(fmaxf(__builtin_rintf(at(j + 1) * inv), -7.0f), 7.0f);
+        dst[(size_t)row * (k >> 1) + (j >> 1)] = (uint8_t)(((int)r0 & 0xF) | (((int)r1 & 0xF) << 4));
+    }
+}
+
+template <int IN>
+static hipError_t launch_quantize_pack(const void *x, void *dst, float *scales, int rows, int k, hipStream_t s)
+{
+    const uint8_t *xb = static_cast<const uint8_t *>(x);
+    uint8_t *db = static_cast<uint8_t *>(dst);
+    const bool vec = k % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)dst & 3) == 0;
+    if (!vec) quantize_pack_scalar_kernel<IN><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
+    else if (k <= 2048 * 2) quantize_pack_kernel<IN, 2><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
+    else if (k <= 2048 * 8) quantize_pack_kernel<IN, 8><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
+    else quantize_pack_kernel<IN, 0><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
+    return hipGetLastError();
+}
+
 static unsigned flat_grid(size_t items, unsigned block)
 {
     size_t g = (items + block - 1) / block;
@@ -483,6 +634,21 @@ QM_EXPORT int qm_pack_i4(const void *src_i8, void *dst_packed, int rows, int k, 
     else
         pack_i4_byte_kernel<<<dim3(flat_grid(nbytes, 256)), dim3(256), 0, s>>>(static_cast<const uint8_t *>(src_i8), static_cast<uint8_t *>(dst_packed), nbytes);
     const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
+QM_EXPORT int qm_quantize_pack_i4(const void *x, int in_dtype, void *dst_packed, float *scales, int rows, int k, void *stream)
+{
+    if (in_dtype != QM_IN_F16 && in_dtype != QM_IN_BF16 && in_dtype != QM_IN_F32) return QM_ERR_DTYPE;
+    if (rows < 0 || k < 0 || (k & 1)) return QM_ERR_SHAPE;
+    if (rows == 0) return QM_OK;
+    if (!scales || (k > 0 && (!x || !dst_packed))) return QM_ERR_NULL;
+    if (((uintptr_t)x & (in_dtype == QM_IN_F32 ? 3 : 1)) || ((uintptr_t)scales & 3)) return QM_ERR_ALIGN;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (in_dtype == QM_IN_F16) e = launch_quantize_pack<QM_IN_F16>(x, dst_packed, scales, rows, k, s);
+    else if (in_dtype == QM_IN_BF16) e = launch_quantize_pack<QM_IN_BF16>(x, dst_packed, scales, rows, k, s);
+    else e = launch_quantize_pack<QM_IN_F32>(x, dst_packed, scales, rows, k, s);
     return e == hipSuccess ? QM_OK : fail_launch(e);
 }
 

@@ -220,3 +220,34 @@ def test_scaled_output_against_numpy_and_torch(oracle_mod):
         assert (one == torch.from_numpy(small).to(tdt).view(torch.int16).numpy().view(np.uint16)).all()
         two = oracle_mod.scale_round16(small, np.full(5, 0.25, np.float32), np.full(7, 8.0, np.float32), out)
         assert (two == (torch.from_numpy(small).to(torch.float32) * 2).to(tdt).view(torch.int16).numpy().view(np.uint16)).all()
+
+
+# ---------------------------------------------------------------- quantise + pack
+def test_quantize_pack_closed_forms(oracle_mod):
+    # a row that already is integers times a power of two quantises to itself
+    q = np.array([[-7, 7, 0, 3, -1, 5, 2, -6]], dtype=np.float32)
+    for s_ in (1.0, 0.25, 8.0):
+        packed, scales = oracle_mod.quantize_pack(q * np.float32(s_))
+        assert scales[0] == np.float32(s_)
+        assert (oracle_mod.unpack_i4(packed)[0] == q[0].astype(np.int8)).all()
+    # ties go to even: amax 7 -> inv 1; 0.5 -> 0, 1.5 -> 2, 2.5 -> 2, -3.5 -> -4, 6.5 -> 6
+    x = np.array([[7, 0.5, 1.5, 2.5, -3.5, 6.5, -0.5, -6.5]], dtype=np.float32)
+    packed, scales = oracle_mod.quantize_pack(x)
+    assert (oracle_mod.unpack_i4(packed)[0] == np.array([7, 0, 2, 2, -4, 6, 0, -6], dtype=np.int8)).all() and scales[0] == 1.0
+    # an all-zero row: zero scale, zero nibbles; the value -8 is never produced
+    packed, scales = oracle_mod.quantize_pack(np.zeros((2, 6), np.float32))
+    assert (packed == 0).all() and (scales == 0).all()
+    x = np.array([[-100.0, 100.0, -99.9, 50.0]], dtype=np.float32)
+    assert oracle_mod.unpack_i4(oracle_mod.quantize_pack(x)[0])[0].min() == -7
+
+
+def test_quantize_pack_against_numpy_and_round_trip(oracle_mod):
+    rng = np.random.default_rng(11)
+    for dt in (np.float16, np.float32):
+        x = (rng.standard_normal((41, 258)) * rng.uniform(0.01, 30, (41, 1))).astype(dt).astype(np.float32)
+        packed, scales = oracle_mod.quantize_pack(x)
+        p2, s2 = oracle_mod.quantize_pack_numpy(x)
+        assert (packed == p2.view(np.uint8)).all() and (scales == s2).all()
+        deq = oracle_mod.unpack_i4(packed).astype(np.float32) * scales[:, None]
+        assert (np.abs(deq - x) <= scales[:, None] * 0.50001 + 1e-30).all()  # within half a step
+        assert (scales == np.abs(x).max(axis=1) / np.float32(7)).all()
