@@ -99,6 +99,25 @@ torch::Tensor pack(torch::Tensor values)
     return out;
 }
 
+// Per-row symmetric int4 quantisation fused with the packing (no counterpart in the
+// reference beyond pack_b's packing half): [rows, K] fp16 / bf16 / fp32 -> ([rows, K/2]
+// int8, [rows] float32 scales = amax / 7, the row_scale of gemm_scaled).
+std::tuple<torch::Tensor, torch::Tensor> quantize_pack(torch::Tensor x)
+{
+    TORCH_CHECK(x.is_cuda() && x.dim() == 2, "quadmul.quantize_pack: expects a 2-D GPU tensor");
+    const auto t = x.scalar_type();
+    TORCH_CHECK(t == torch::kFloat16 || t == torch::kBFloat16 || t == torch::kFloat32, "quadmul.quantize_pack: x must be float16, bfloat16 or float32");
+    TORCH_CHECK(x.size(1) % 2 == 0, "quadmul.quantize_pack: K must be even");
+    auto v = x.contiguous();
+    c10::OptionalDeviceGuard guard(v.device());
+    auto packed = torch::empty({v.size(0), v.size(1) / 2}, v.options().dtype(torch::kInt8));
+    auto scales = torch::empty({v.size(0)}, v.options().dtype(torch::kFloat32));
+    const int in = t == torch::kFloat16 ? QM_IN_F16 : (t == torch::kBFloat16 ? QM_IN_BF16 : QM_IN_F32);
+    check_status(qm_quantize_pack_i4(v.data_ptr(), in, packed.data_ptr(), scales.data_ptr<float>(), (int)v.size(0), (int)v.size(1), stream_of(v)),
+                 "quadmul.quantize_pack");
+    return {packed, scales};
+}
+
 // Device-side unpack_int4_matrix (kernel.cu:389-408): [rows, K/2] bytes -> [rows, K] int8.
 torch::Tensor unpack(torch::Tensor packed)
 {
@@ -149,6 +168,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
           py::arg("d"), py::arg("m"), py::arg("n"), py::arg("k"), py::arg("row_scale") = py::none(), py::arg("col_scale") = py::none());
     m.def("gemm_cfg", &gemm_cfg, "gemm with an explicit kernel configuration id (autotuning)");
     m.def("pack", &pack, "Pack a [rows, K] int8 tensor of int4 values into [rows, K/2] bytes on the GPU");
+    m.def("quantize_pack", &quantize_pack, "Per-row symmetric int4 quantisation of a [rows, K] float tensor, packed; returns (packed, scales)");
     m.def("unpack", &unpack, "Unpack [rows, K/2] bytes into a [rows, K] int8 tensor on the GPU");
     m.def("num_configs", &qm_num_configs);
     m.def("config_name", [](int cfg) { const char *s = qm_config_name(cfg); return std::string(s ? s : ""); });

@@ -57,8 +57,10 @@ def test_int4_linear_layer_end_to_end(oracle_mod):
     g = torch.Generator().manual_seed(SEED_BASE + 8200)
     x = (torch.randn((m, k), generator=g) * 0.5).to(torch.float16)
     w = (torch.randn((n, k), generator=g) * 0.05).to(torch.float16)
-    xq, xs = qm.quantize_pack(x.to(DEV))
-    wq, ws = qm.quantize_pack(w.to(DEV))
+    import quadmul
+
+    xq, xs = quadmul.quantize_pack(x.to(DEV))   # the extension module's entry point
+    wq, ws = qm.quantize_pack(w.to(DEV))        # the ctypes binding of the same C function
     y = torch.empty((m, n), dtype=torch.float16, device=DEV)
     qm.gemm_scaled(xq, wq, y, m, n, k, xs, ws)
     torch.cuda.synchronize()
