@@ -11,15 +11,32 @@
 //     16x16x64 int8 MFMA sustains a clearly higher rate than the 32x32x32 one, and
 //     operands of the form 16*s4 (low nibble zero) are cheaper than sign-extended.
 //   * LDS holds the packed bytes (half the LDS traffic of an int8 tile); each wave
-//     widens its own fragments after ds_read: 3 VALU instructions per dword.
+//     widens its own fragments after ds_read: 10 VALU instructions per 16 bytes.
 //   * Tiles travel global -> LDS without touching registers (global_load_lds, 16
-//     bytes per lane): no staging registers, no ds_write.  Ring of 4 stages: while
-//     tile t is contracted, B fragments of tile t+1 are read and widened, tile t+2
-//     has landed and tile t+3 is in flight; one barrier per K-step.
+//     bytes per lane): no staging registers, no ds_write.  Ring of 3 to 5 stages
+//     (4 by default): while step s is contracted, B fragments of step s+1 are read
+//     and widened, step s+2 has landed and step s+3 is in flight; one barrier per
+//     K-step.
 //   * The compiler's scheduler, left alone, puts the two MFMAs that update one
 //     accumulator back to back and bunches the VALU work, which stalls the matrix
 //     pipe.  The K-step is therefore written slot by slot -- one MFMA plus its share
 //     of reads / widening / DMA -- with a scheduling barrier after every slot.
+//   * The grid is persistent: a workgroup runs its tiles as one stream of K-steps,
+//     the loads running ahead through tile boundaries, and the write-out of a whole
+//     tile rides in the MFMA slots of its last K-step, through a per-wave LDS
+//     transpose where there is room, so that stores cover contiguous row segments.
+//   * Outputs: the exact int32 product, or (template parameter OUT) the product
+//     scaled per row and per column in fp32 and rounded to fp16 / bf16.
+//
+// Rules the code keeps, each learnt from a wrong result or a slow kernel:
+//   * the accumulators are read, written and cleared through asm statements only,
+//     by one set of statements on every path (else the register allocator copies
+//     all of them around);
+//   * no per-lane branch inside the slot code of a K-step (selects instead);
+//   * every lambda is always_inline (an outlined one takes all state to memory);
+//   * values an asm statement writes into registers that a 16-byte store or
+//     ds_write just before may still be reading get two wait states first (the
+//     compiler pads that hazard only for instructions it can see).
 #pragma once
 #include <type_traits>
 
