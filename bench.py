@@ -232,7 +232,8 @@ def main(argv=None):
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="square4096", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="square4096", choices=sorted(WORKLOADS) + ["square4096_scaled_f16", "quantize4096_f16"],
+                    help="the workload of the JSON line; the last two names exist for --launches-only (profiling) only")
     ap.add_argument("--no-targets", action="store_true", help="skip the other target shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--launches-only", type=int, default=0, metavar="N",
@@ -259,6 +260,31 @@ def main(argv=None):
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"bytes_read_per_copy": 256 << 20, "bytes_written_per_copy": 256 << 20, "copies": 10}}))
         return 0
+    if a.launches_only and a.workload == "quantize4096_f16":
+        import quadmul
+
+        x = torch.randn((4096, 4096), device="cuda:0").to(torch.float16)
+        for _ in range(a.launches_only + 1):
+            quadmul.quantize_pack(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"launches_only": a.launches_only, "workload": a.workload}))
+        return 0
+    if a.launches_only and a.workload == "square4096_scaled_f16":
+        import quadmul
+
+        row, m, n, k, _ = WORKLOADS["square4096"]
+        apk, bpk = make_packed(m, n, k, SEED_BASE + row)
+        a_d, b_d = apk.to("cuda:0"), bpk.to("cuda:0")
+        d_d = torch.empty((m, n), dtype=torch.float16, device="cuda:0")
+        rs, cs = torch.rand(m, device="cuda:0") * 0.02 + 1e-3, torch.rand(n, device="cuda:0") * 0.05 + 1e-4
+        for _ in range(a.launches_only + 1):
+            quadmul.gemm_scaled(a_d, b_d, d_d, m, n, k, rs, cs)
+        torch.cuda.synchronize()
+        print(json.dumps({"launches_only": a.launches_only, "workload": a.workload}))
+        return 0
+    if a.workload not in WORKLOADS:
+        print("bench.py: that workload name is for --launches-only", file=sys.stderr)
+        return 2
     if a.launches_only:
         import quadmul
 
@@ -286,6 +312,17 @@ def main(argv=None):
     }
     if "scaled_fp16_output" in main_res:
         line["scaled_fp16_output"] = main_res["scaled_fp16_output"]
+    if a.workload == "square4096":
+        # the step before the GEMM: quantise + pack a [4096, 4096] fp16 activation matrix (HBM-bound)
+        import quadmul
+        x = torch.randn((m, k), device="cuda:0").to(torch.float16)
+        q_ms = time_graph(lambda: quadmul.quantize_pack(x), launches=50)
+        q_bytes = m * k * 2 + m * k // 2 + 4 * m
+        line["quantize_pack_fp16"] = {"entry_point": "quadmul.quantize_pack(x)", "rows": m, "k": k, "ms_per_launch_graph": round(q_ms, 5),
+                                      "algorithmic_bytes": q_bytes,
+                                      "roofline": {"bound": "hbm", "achieved": round(q_bytes / q_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                                   "frac": round(q_bytes / q_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}}
+        del x
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(apk, bpk, c_d, m, n, k)
     del apk, bpk, c_d

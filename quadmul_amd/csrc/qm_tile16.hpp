@@ -616,6 +616,11 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 });
             });
         }
+        // The clearing MFMAs issued last must have retired before anything else touches the
+        // accumulators: between the two loops below the register allocator may move
+        // accumulators to other registers with instructions of its own, and it does not know
+        // that asm statements are still writing them.
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     };
     for (; c_item < nwhole; c_item += G) run_item(std::true_type{});
     for (; c_item < nitems; c_item += G) run_item(std::false_type{});
