@@ -74,7 +74,23 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
     assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
     assert lib.qm_unpack_i4(None, one, 4, 8, None) == -1
-    for code in (0, -1, -2, -3, -4, -5):
+    # the scaled GEMM and the quantiser reject bad arguments before they touch the GPU too
+    assert lib.qm_gemm_i4_scaled(one, one, one, 4, 4, 4, None, None, 7, None) == -6        # unknown output type
+    assert lib.qm_gemm_i4_scaled(one, one, one, 4, 4, 3, None, None, 1, None) == -2
+    assert lib.qm_gemm_i4_scaled(one, one, None, 4, 4, 4, None, None, 1, None) == -1
+    assert lib.qm_gemm_i4_scaled(one, one, ctypes.c_void_p(4097), 4, 4, 4, None, None, 2, None) == -5
+    assert lib.qm_gemm_i4_scaled(None, None, None, 0, 4, 4, None, None, 1, None) == 0
+    assert lib.qm_gemm_i4_scaled_cfg(one, one, one, 64, 64, 128, None, None, 1, None, qm.config_id("t64x64x128_w2x2_m0")) == -3
+    assert lib.qm_gemm_i4_scaled_cfg(one, one, one, 256, 256, 256, None, None, 1, None, qm.config_id("q256x256_w2x2_s4o1") | (2 << 24)) == -3
+    assert lib.qm_quantize_pack_i4(one, 9, one, one, 4, 8, None) == -6
+    assert lib.qm_quantize_pack_i4(one, 1, one, one, 4, 7, None) == -2
+    assert lib.qm_quantize_pack_i4(one, 1, one, None, 4, 8, None) == -1
+    assert lib.qm_quantize_pack_i4(ctypes.c_void_p(4097), 1, one, one, 4, 8, None) == -5
+    assert lib.qm_quantize_pack_i4(None, 3, None, None, 0, 8, None) == 0
+    has = [qm.config_has_scaled(i) for i in range(qm.num_configs())]
+    assert has[qm.config_id("generic")] and has[qm.config_id("q256x256_w2x2_s4o1")] and has[qm.config_id("s1x1_w8_u4")]
+    assert not has[qm.config_id("t64x64x128_w2x2_m0")] and not has[qm.config_id("q256x128_w2x2_s3o2")]
+    for code in (0, -1, -2, -3, -4, -5, -6):
         assert lib.qm_status_string(code)
     assert b"gfx950" in lib.qm_version()
 
