@@ -105,7 +105,8 @@ def time_graph(fn, launches=200, replays=5):
 # Bytes moved per launch past the L2s, from rocprofv3 counter runs of `bench.py --workload W
 # --launches-only 20` (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads
 # for a 256 MiB device-to-device copy; summaries under profiles/).  Not measured live.
-MEASURED_TRAFFIC = {(4096, 4096, 4096): 118968897, (8192, 8192, 8192): 677105932, (16, 4096, 4096): 8961456}
+MEASURED_TRAFFIC = {(4096, 4096, 4096): 118980616, (8192, 8192, 8192): 677216905, (16, 4096, 4096): 8953239}
+MEASURED_TRAFFIC_OTHER = {"scaled_fp16_4096^3": 84831911, "quantize_pack_fp16_4096x4096": 42116604}
 
 
 def roofline_of(m, n, k, bound, ms):
@@ -184,6 +185,7 @@ def run_workload(name, steps, warmup, check_rows=64):
                                      "ms_per_launch_graph": round(scaled_ms, 5), "tops": round(2.0 * m * n * k / scaled_ms / 1e9, 1),
                                      "frac_of_int8_peak": round(2.0 * m * n * k / scaled_ms / 1e9 / INT8_PEAK_TOPS, 4),
                                      "algorithmic_bytes": m * k // 2 + n * k // 2 + 2 * m * n + 4 * (m + n),
+                                     "traffic": MEASURED_TRAFFIC_OTHER["scaled_fp16_4096^3"],
                                      "checked": "every element against torch's float32 arithmetic on the int32 result"}
     if rotating_ms is not None:
         out["ms_per_launch_graph_rotating_b"] = round(rotating_ms, 5)
@@ -321,7 +323,8 @@ def main(argv=None):
         line["quantize_pack_fp16"] = {"entry_point": "quadmul.quantize_pack(x)", "rows": m, "k": k, "ms_per_launch_graph": round(q_ms, 5),
                                       "algorithmic_bytes": q_bytes,
                                       "roofline": {"bound": "hbm", "achieved": round(q_bytes / q_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                                   "frac": round(q_bytes / q_ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}}
+                                                   "frac": round(q_bytes / q_ms / 1e6 / HBM_PEAK_GBS, 4),
+                                                   "traffic": MEASURED_TRAFFIC_OTHER["quantize_pack_fp16_4096x4096"]}}
         del x
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(apk, bpk, c_d, m, n, k)

@@ -25,6 +25,7 @@
 #define QM_ABI_H
 
 #include <stdint.h>
+#include <stddef.h>
 
 #ifdef __cplusplus
 extern "C" {
@@ -87,9 +88,36 @@ int qm_gemm_i4_scaled_cfg(const void *A, const void *B, void *D, int m, int n, i
                           const float *col_scale, int out_dtype, void *stream, int cfg);
 int qm_config_has_scaled(int cfg); /* 1 / 0 */
 
-/* The configuration qm_gemm_i4 would pick for this shape (the table lookup the
- * reference does at kernel.cu:340-385, here with a heuristic fallback instead of
- * a silent no-op).  ptr_align is the smallest alignment in bytes shared by A and
+/*
+ * The two GEMMs with a caller-provided workspace (the counterpart of the workspace
+ * argument of vendor GEMM libraries; the reference's wrapper, kernel.cu:334, has none
+ * because its kernels never split K).  Shapes with few output tiles and a long K run
+ * faster with K split over several workgroups per tile; with a workspace each split
+ * stores its partial tile there with plain 16-byte stores and a second kernel adds the
+ * splits up (scaling and rounding, for the scaled form), instead of 4-byte atomics into
+ * C.  Results are identical to the forms without a workspace.
+ *   workspace        device memory, 16-byte aligned, or NULL; used by the kernels of this
+ *                    call only (in stream order): calls that may overlap on the GPU need
+ *                    a workspace each, calls on one stream can share one
+ *   workspace_bytes  its size; qm_gemm_workspace_bytes says how much this call can use.
+ *                    A smaller (or no) workspace is not an error: the call then runs as
+ *                    the form without one (except that an explicit cfg with a K split
+ *                    and the scaled output returns QM_ERR_CONFIG).
+ * cfg as for qm_gemm_i4_cfg (QM_CFG_AUTO included); with a workspace the scaled form also
+ * takes K splits, on every "q" configuration.
+ * qm_gemm_workspace_bytes: what the call with these arguments uses at most (0 when it
+ * would not split K); scaled = 1 for the scaled form.
+ */
+int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg,
+                  void *workspace, size_t workspace_bytes);
+int qm_gemm_i4_scaled_ws(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
+                         const float *col_scale, int out_dtype, void *stream, int cfg, void *workspace,
+                         size_t workspace_bytes);
+size_t qm_gemm_workspace_bytes(int m, int n, int k, int ptr_align, int cfg, int scaled);
+
+/* The configuration qm_gemm_i4_ws picks for this shape when it is given a workspace
+ * (the table lookup the reference does at kernel.cu:340-385, here with a heuristic
+ * fallback instead of a silent no-op); without a workspace the K split may be lower.  ptr_align is the smallest alignment in bytes shared by A and
  * B (pass 16 or more when they come from a device allocator). */
 int qm_select_config(int m, int n, int k, int ptr_align);
 

@@ -34,7 +34,8 @@ _lib: Optional[ctypes.CDLL] = None
 CFG_AUTO = -1
 #: every symbol include/qm_abi.h declares
 ABI_SYMBOLS = (
-    "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled", "qm_quantize_pack_i4", "qm_select_config", "qm_num_configs", "qm_config_name",
+    "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled",
+    "qm_gemm_i4_ws", "qm_gemm_i4_scaled_ws", "qm_gemm_workspace_bytes", "qm_quantize_pack_i4", "qm_select_config", "qm_num_configs", "qm_config_name",
     "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version",
 )
 
@@ -66,6 +67,12 @@ def library() -> ctypes.CDLL:
     lib.qm_gemm_i4_scaled.restype = ci
     lib.qm_gemm_i4_scaled_cfg.argtypes = [vp, vp, vp, ci, ci, ci, vp, vp, ci, vp, ci]
     lib.qm_gemm_i4_scaled_cfg.restype = ci
+    lib.qm_gemm_i4_ws.argtypes = [vp, vp, vp, ci, ci, ci, vp, ci, vp, ctypes.c_size_t]
+    lib.qm_gemm_i4_ws.restype = ci
+    lib.qm_gemm_i4_scaled_ws.argtypes = [vp, vp, vp, ci, ci, ci, vp, vp, ci, vp, ci, vp, ctypes.c_size_t]
+    lib.qm_gemm_i4_scaled_ws.restype = ci
+    lib.qm_gemm_workspace_bytes.argtypes = [ci, ci, ci, ci, ci, ci]
+    lib.qm_gemm_workspace_bytes.restype = ctypes.c_size_t
     lib.qm_config_has_scaled.argtypes = [ci]
     lib.qm_config_has_scaled.restype = ci
     lib.qm_quantize_pack_i4.argtypes = [vp, ci, vp, vp, ci, ci, vp]
@@ -128,24 +135,57 @@ def _check_operands(a, b, c, m, n, k, c_dtypes=(torch.int32,)) -> None:
         raise QuadmulError("gemm: tensor sizes do not match m, n, k")
 
 
-def gemm_cfg(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int, cfg: int = CFG_AUTO) -> None:
+def _ptr_align(*tensors) -> int:
+    x = 0
+    for t in tensors:
+        x |= t.data_ptr()
+    return 4096 if x == 0 else min(x & -x, 4096)
+
+
+def workspace_bytes(m: int, n: int, k: int, cfg: int = CFG_AUTO, scaled: bool = False, ptr_align: int = 256) -> int:
+    """Bytes of workspace the GEMM of this shape can use (0: it would not split K)."""
+    return int(library().qm_gemm_workspace_bytes(m, n, k, ptr_align, cfg, 1 if scaled else 0))
+
+
+def _workspace(workspace, a, b, m, n, k, cfg, scaled):
+    """(pointer, bytes, keep-alive) of the workspace argument: True = allocate what the call
+    can use from torch's caching allocator (stream-ordered, so safe across streams and under
+    graph capture), None / False = none, a tensor = the caller's own."""
+    if workspace is None or workspace is False:
+        return None, 0, None
+    if workspace is True:
+        need = workspace_bytes(m, n, k, cfg, scaled, _ptr_align(a, b))
+        if need == 0:
+            return None, 0, None
+        workspace = torch.empty((need,), dtype=torch.uint8, device=a.device)
+    if not (isinstance(workspace, torch.Tensor) and workspace.is_cuda and workspace.device == a.device and workspace.is_contiguous()):
+        raise QuadmulError("gemm: workspace must be a contiguous tensor on a's device")
+    return workspace.data_ptr(), workspace.numel() * workspace.element_size(), workspace
+
+
+def gemm_cfg(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int, cfg: int = CFG_AUTO,
+             workspace=True) -> None:
     """``c[m,n] = a[m,k] @ b[n,k].T`` on packed int4, with an explicit kernel configuration.
 
     ``cfg``: config id in the low 16 bits, tile-raster group height in bits 16..23
-    (0 = default); ``CFG_AUTO`` = table / cost model.
+    (0 = default), K split in bits 24..29; ``CFG_AUTO`` = table / cost model.
+    ``workspace``: see :func:`gemm`.
     """
     _check_operands(a, b, c, m, n, k)
+    ws, ws_bytes, _keep = _workspace(workspace, a, b, m, n, k, cfg, False)
     with torch.cuda.device(a.device):
-        st = library().qm_gemm_i4_cfg(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, _stream_ptr(a), cfg)
-    _check(st, "qm_gemm_i4_cfg")
+        st = library().qm_gemm_i4_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, _stream_ptr(a), cfg, ws, ws_bytes)
+    _check(st, "qm_gemm_i4_ws")
 
 
 def gemm_scaled(a: torch.Tensor, b: torch.Tensor, d: torch.Tensor, m: int, n: int, k: int,
-                row_scale: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None, cfg: int = CFG_AUTO) -> None:
+                row_scale: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None, cfg: int = CFG_AUTO,
+                workspace=True) -> None:
     """The GEMM with the dequantising epilogue fused in (no counterpart in the reference's
     code; README.md:7 names the idea): ``d[m,n] = round(((float)c[m,n] * row_scale[m]) *
     col_scale[n])`` with ``c`` the exact int32 product; ``d`` is float16 or bfloat16 and is
-    overwritten; the scales are float32 vectors on the same device, None = all ones."""
+    overwritten; the scales are float32 vectors on the same device, None = all ones.
+    ``workspace``: see :func:`gemm`."""
     _check_operands(a, b, d, m, n, k, c_dtypes=(torch.float16, torch.bfloat16))
     for s_, cnt, what in ((row_scale, m, "row_scale"), (col_scale, n, "col_scale")):
         if s_ is None:
@@ -153,11 +193,13 @@ def gemm_scaled(a: torch.Tensor, b: torch.Tensor, d: torch.Tensor, m: int, n: in
         if not (s_.is_cuda and s_.device == a.device and s_.dtype == torch.float32 and s_.is_contiguous() and s_.numel() == cnt):
             raise QuadmulError(f"gemm_scaled: {what} must be a contiguous float32 vector of {cnt} elements on a's device")
     out = 1 if d.dtype == torch.float16 else 2
+    ws, ws_bytes, _keep = _workspace(workspace, a, b, m, n, k, cfg, True)
     with torch.cuda.device(a.device):
-        st = library().qm_gemm_i4_scaled_cfg(a.data_ptr(), b.data_ptr(), d.data_ptr(), m, n, k,
-                                             None if row_scale is None else row_scale.data_ptr(),
-                                             None if col_scale is None else col_scale.data_ptr(), out, _stream_ptr(a), cfg)
-    _check(st, "qm_gemm_i4_scaled")
+        st = library().qm_gemm_i4_scaled_ws(a.data_ptr(), b.data_ptr(), d.data_ptr(), m, n, k,
+                                            None if row_scale is None else row_scale.data_ptr(),
+                                            None if col_scale is None else col_scale.data_ptr(), out, _stream_ptr(a), cfg,
+                                            ws, ws_bytes)
+    _check(st, "qm_gemm_i4_scaled_ws")
 
 
 def quantize_pack(x: torch.Tensor):
@@ -186,14 +228,16 @@ def config_has_scaled(cfg: int) -> bool:
     return bool(library().qm_config_has_scaled(cfg))
 
 
-def gemm(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int) -> None:
+def gemm(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int, workspace=True) -> None:
     """Same contract as the reference's ``quadmul.gemm`` (extension.cpp:8-24): ``a`` is
     packed A ``[m, k/2]``, ``b`` is packed B stored ``[n, k/2]``, ``c`` is ``[m, n]`` int32
-    and is overwritten; enqueued on the current stream of ``a``'s device; returns None."""
-    _check_operands(a, b, c, m, n, k)
-    with torch.cuda.device(a.device):
-        st = library().qm_gemm_i4(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, _stream_ptr(a))
-    _check(st, "qm_gemm_i4")
+    and is overwritten; enqueued on the current stream of ``a``'s device; returns None.
+
+    ``workspace``: True (default) takes a temporary buffer from torch's allocator when the
+    shape runs with K split over several workgroups per tile (few tiles, long K); None runs
+    without one (the splits then meet in ``c`` through atomics); a uint8 tensor is used as
+    it is.  The result is the same in every case."""
+    gemm_cfg(a, b, c, m, n, k, CFG_AUTO, workspace)
 
 
 def pack_int4(values: torch.Tensor) -> torch.Tensor:

@@ -120,7 +120,7 @@ def tune_shape(m: int, n: int, k: int, device, group_ms: Iterable[int], min_ms: 
         if name[0] == "q":
             bm, bn = (int(x) for x in name[1:].split("_")[0].split("x"))
             tiles = -(-m // bm) * -(-n // bn)
-            kss = [ks for ks in (1, 2, 4, 8) if ks == 1 or (tiles * ks <= 512 and (k // 128) // ks >= 4)]
+            kss = [ks for ks in (1, 2, 3, 4, 6, 8, 12, 16) if ks == 1 or (tiles * ks <= 1024 and tiles <= 256 and (k // 128) // ks >= 4)]
         # (K split, group height, one-item-per-workgroup flag); the flag only changes the launch
         # when there are more work items than the device holds workgroups of the pipelined kernel
         variants = [(g_, k_, 0) for k_ in kss for g_ in (gms if k_ == 1 else gms[:1])]

@@ -49,11 +49,32 @@ void check_operands(const torch::Tensor &a, const torch::Tensor &b, const torch:
     TORCH_CHECK(c.numel() == m * n, "quadmul.gemm: c must hold m*n int32, got ", c.numel());
 }
 
+// The workspace of a call that splits K (few output tiles, long K), from torch's caching
+// allocator: stream-ordered, so calls on different streams never share one, and legal under
+// graph capture.  An undefined tensor when the shape does not split.
+int ptr_alignment(const torch::Tensor &a, const torch::Tensor &b)
+{
+    const uintptr_t x = reinterpret_cast<uintptr_t>(a.data_ptr()) | reinterpret_cast<uintptr_t>(b.data_ptr());
+    if (x == 0) return 4096;
+    const uintptr_t low = x & (~x + 1);
+    return low > 4096 ? 4096 : (int)low;
+}
+
+torch::Tensor workspace_for(const torch::Tensor &a, const torch::Tensor &b, int64_t m, int64_t n, int64_t k, int cfg, bool scaled)
+{
+    const size_t need = qm_gemm_workspace_bytes((int)m, (int)n, (int)k, ptr_alignment(a, b), cfg, scaled ? 1 : 0);
+    if (need == 0) return torch::Tensor();
+    return torch::empty({(int64_t)need}, a.options().dtype(torch::kUInt8));
+}
+
 void gemm(torch::Tensor a, torch::Tensor b, torch::Tensor c, int64_t m, int64_t n, int64_t k)
 {
     check_operands(a, b, c, m, n, k);
     c10::OptionalDeviceGuard guard(a.device());
-    check_status(qm_gemm_i4(a.data_ptr(), b.data_ptr(), c.data_ptr(), (int)m, (int)n, (int)k, stream_of(a)), "quadmul.gemm");
+    const torch::Tensor ws = workspace_for(a, b, m, n, k, QM_CFG_AUTO, false);
+    check_status(qm_gemm_i4_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), (int)m, (int)n, (int)k, stream_of(a), QM_CFG_AUTO,
+                               ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0),
+                 "quadmul.gemm");
 }
 
 // The GEMM with the dequantising epilogue fused in (no counterpart in the reference's code;
@@ -74,9 +95,11 @@ void gemm_scaled(torch::Tensor a, torch::Tensor b, torch::Tensor d, int64_t m, i
     check_scale(col_scale, a, n, "col_scale");
     c10::OptionalDeviceGuard guard(a.device());
     const int out = d.scalar_type() == torch::kFloat16 ? QM_OUT_F16 : QM_OUT_BF16;
-    check_status(qm_gemm_i4_scaled(a.data_ptr(), b.data_ptr(), d.data_ptr(), (int)m, (int)n, (int)k,
-                                   row_scale.has_value() ? row_scale->data_ptr<float>() : nullptr,
-                                   col_scale.has_value() ? col_scale->data_ptr<float>() : nullptr, out, stream_of(a)),
+    const torch::Tensor ws = workspace_for(a, b, m, n, k, QM_CFG_AUTO, true);
+    check_status(qm_gemm_i4_scaled_ws(a.data_ptr(), b.data_ptr(), d.data_ptr(), (int)m, (int)n, (int)k,
+                                      row_scale.has_value() ? row_scale->data_ptr<float>() : nullptr,
+                                      col_scale.has_value() ? col_scale->data_ptr<float>() : nullptr, out, stream_of(a), QM_CFG_AUTO,
+                                      ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0),
                  "quadmul.gemm_scaled");
 }
 
@@ -84,7 +107,10 @@ void gemm_cfg(torch::Tensor a, torch::Tensor b, torch::Tensor c, int64_t m, int6
 {
     check_operands(a, b, c, m, n, k);
     c10::OptionalDeviceGuard guard(a.device());
-    check_status(qm_gemm_i4_cfg(a.data_ptr(), b.data_ptr(), c.data_ptr(), (int)m, (int)n, (int)k, stream_of(a), (int)cfg), "quadmul.gemm_cfg");
+    const torch::Tensor ws = workspace_for(a, b, m, n, k, (int)cfg, false);
+    check_status(qm_gemm_i4_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), (int)m, (int)n, (int)k, stream_of(a), (int)cfg,
+                               ws.defined() ? ws.data_ptr() : nullptr, ws.defined() ? (size_t)ws.numel() : 0),
+                 "quadmul.gemm_cfg");
 }
 
 // Device-side pack_b (test.py:6-15): [rows, K] int8 -> [rows, K/2] int8.

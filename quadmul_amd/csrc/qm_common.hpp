@@ -23,6 +23,11 @@ struct GemmArgs {
     const float *row_scale = nullptr;  // [M]
     const float *col_scale = nullptr;  // [N]
     int out = OUT_I32;
+    // K split over several work items per tile (pipelined kernel): where the partial sums go.
+    // Null: they meet in C by atomic adds (C zero-filled beforehand).  Otherwise item i of the
+    // launch stores its tile here, 16 bytes per lane in the order the MFMA leaves them, and a
+    // second kernel adds the splits up.
+    int32_t *ws = nullptr;
 };
 
 __device__ __forceinline__ float scale_at(const float *s, int i, int n) { return (s != nullptr && i < n) ? s[i] : 1.0f; }

@@ -76,6 +76,88 @@ __global__ void fill_zero_kernel(int32_t *dst, size_t n)
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = 0;
 }
 
+// --------------------------------------------------------------------------
+// K split with a workspace (pipelined kernel): item (split s, tile t) of the GEMM launch
+// left its BM x BN partial sums in slot s * ntiles + t, wave by wave, block by block, 16
+// bytes per lane in the order the MFMA leaves a block (lane l: row l % 16, columns
+// 4 * (l / 16) .. + 3).  One thread here adds up the splits of one such 16-byte piece and
+// stores the four sums -- as int32, or scaled and rounded to a 16-bit float -- with the
+// guards of the matrix edge.  Tiles are numbered as the GEMM kernel numbers them (columns of
+// group_m tiles).
+// --------------------------------------------------------------------------
+struct SplitReduceArgs {
+    const v4i *ws;
+    void *C;
+    int M, N;
+    int tiles_m, tiles_n, group_m, ksplit;
+    int BM, BN, WGN, FM, FN, waves;
+    const float *row_scale, *col_scale;
+    int out;
+};
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitReduceArgs q)
+{
+    const int blocks = q.FM * q.FN;
+    const size_t per_tile = (size_t)q.waves * blocks * 64;  // 16-byte pieces per slot
+    const size_t ntiles = (size_t)q.tiles_m * q.tiles_n;
+    const uint32_t t = blockIdx.x * 256u + threadIdx.x;  // (the launcher keeps the count below 2^31)
+    if (t >= ntiles * per_tile) return;
+    const v4i *src = q.ws + t;
+    const size_t stride = ntiles * per_tile;
+    v4i sum = {0, 0, 0, 0};
+    // four splits at a time, so that their loads are in flight together (splits past the
+    // last re-read it and count for nothing)
+    for (int s = 0; s < q.ksplit; s += 4) {
+        v4i v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __builtin_nontemporal_load(src + (size_t)min(s + i, q.ksplit - 1) * stride);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int on = s + i < q.ksplit ? -1 : 0;
+            sum.x += v[i].x & on; sum.y += v[i].y & on; sum.z += v[i].z & on; sum.w += v[i].w & on;
+        }
+    }
+    const int lane = (int)(t & 63);
+    uint32_t u = t >> 6;
+    const int blk = (int)(u % (uint32_t)blocks);
+    u /= (uint32_t)blocks;
+    const int wave = (int)(u % (uint32_t)q.waves);
+    const int pid = (int)(u / (uint32_t)q.waves);
+    const int width = q.group_m * q.tiles_n;
+    const int first_m = (pid / width) * q.group_m;
+    const int gsz = min(q.tiles_m - first_m, q.group_m);
+    const int tm = first_m + (pid % width) % gsz, tn = (pid % width) / gsz;
+    const int m = tm * q.BM + (wave / q.WGN) * q.FM * 16 + (blk / q.FN) * 16 + (lane & 15);
+    const int n = tn * q.BN + (wave % q.WGN) * q.FN * 16 + (blk % q.FN) * 16 + (lane >> 4) * 4;
+    if (m >= q.M || n >= q.N) return;
+    if (q.out == OUT_I32) {
+        int32_t *crow = static_cast<int32_t *>(q.C) + (size_t)m * q.N;
+        if ((q.N & 3) == 0 && ((uintptr_t)q.C & 15) == 0) {
+            *reinterpret_cast<v4i *>(crow + n) = sum;  // n % 4 == 0 and N % 4 == 0: all four inside
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < q.N) crow[n + e] = sum[e];
+        }
+    } else {
+        uint16_t *drow = static_cast<uint16_t *>(q.C) + (size_t)m * q.N;
+        const float rs = scale_at(q.row_scale, m, q.M);
+        uint16_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int c = sum[e];
+            h[e] = round16(scaled(c, rs, scale_at(q.col_scale, n + e, q.N)), q.out);
+        }
+        if ((q.N & 3) == 0 && ((uintptr_t)q.C & 7) == 0) {
+            *reinterpret_cast<v2i *>(drow + n) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < q.N) drow[n + e] = h[e];
+        }
+    }
+}
+
 // 16 int8 in -> 8 packed bytes out per thread when aligned, else one byte per thread.
 __device__ __forceinline__ uint32_t pack4(uint32_t w)  // 4 int8 -> 2 packed bytes in bits 0..15
 {
@@ -314,6 +396,7 @@ struct ConfigDesc {
     int bm, bn, bk;  // tile: block shape; skinny: bm = max M, bn = columns per workgroup
     int waves, mode;
     LaunchFn launch;
+    int wgm = 0, wgn = 0;  // pipelined kernel: waves down and across the tile
 };
 
 #define QM_STR2(x) #x
@@ -325,7 +408,7 @@ static const ConfigDesc g_configs[] = {
      KIND_TILE, BM, BN, BK, (WGM) * (WGN), MODE, &QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)},
 #define QM_TILE16(tu, BM, BN, WGM, WGN, ST, OCC)                                                              \
     {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_s" QM_STR(ST) "o" QM_STR(OCC), KIND_TILE16, BM, BN, 128, \
-     (WGM) * (WGN), 0, &QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)},
+     (WGM) * (WGN), 0, &QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC), WGM, WGN},
 #define QM_SKINNY(FM, FN, NW, U)                                                     \
     {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
      &QM_SKINNY_FN(FM, FN, NW, U)},
@@ -400,7 +483,7 @@ struct Choice {
     int spread = 0;
 };
 
-static Choice heuristic(int m, int n, int k, int ptr_align)
+static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
 {
     if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
     if (m <= 64) {
@@ -423,22 +506,35 @@ static Choice heuristic(int m, int n, int k, int ptr_align)
         if (id < 0 || !config_supports(id, m, n, k, ptr_align)) continue;
         const ConfigDesc &d = g_configs[id];
         const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
-        // Few tiles and a very long K: the pipelined kernel can split K over several
-        // workgroups per tile.  The partial sums meet in C through 4-byte atomics, which
-        // are slow enough that this only pays when each split keeps a long K of its own
+        // Few tiles and a long K: the pipelined kernel can split K over several workgroups
+        // per tile.  With a workspace the partial sums cost a second kernel (about 8 us all
+        // told, measured); without one they meet in C through 4-byte atomics, which are slow
+        // enough that splitting only pays when each split keeps a long K of its own
         // (measured: wins at K = 28672, loses at K = 8192).
+        // Cost in units of 16.5 ps (one K-step of the 256 x 256 tile = 65536): K-steps per
+        // item x tile area / efficiency, plus 3 us per round of workgroups for filling the
+        // ring and writing out, plus the split's own cost.
+        const int kt = (k + 127) / 128;
+        auto cost_of = [&](int ks_) {
+            const long long rounds = (tiles * ks_ + 255) / 256;
+            return (double)rounds * ((double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + 180000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
+        };
         int ks = 1;
-        if (d.kind == KIND_TILE16)
+        double cost = cost_of(1);
+        if (d.kind == KIND_TILE16 && has_ws) {
+            for (int t = 2; t <= 16 && tiles * t <= 256 && kt / t >= 4; ++t)
+                if (cost_of(t) < cost) { cost = cost_of(t); ks = t; }
+        } else if (d.kind == KIND_TILE16) {
             while (ks < 4 && tiles * ks * 2 <= 256 && (k / 128) / (ks * 2) >= 48) ks *= 2;
-        const long long rounds = (tiles * ks + 255) / 256;
-        const double cost = (double)rounds * d.bm * d.bn / c.eff / ks * (ks > 1 ? 1.25 : 1.0);
+            if (ks > 1) cost = (double)d.bm * d.bn / c.eff * ((kt + ks - 1) / ks) * 1.25 + 180000.0;
+        }
         if (cost < best_cost) { best_cost = cost; best = id; best_ks = ks; }
     }
     const int ksplit = best_ks;
     return {best, 4, ksplit};
 }
 
-static Choice select_config(int m, int n, int k, int ptr_align)
+static Choice select_config(int m, int n, int k, int ptr_align, bool has_ws)
 {
     static int resolved[sizeof(g_table) / sizeof(g_table[0])];
     static std::once_flag once;
@@ -449,16 +545,19 @@ static Choice select_config(int m, int n, int k, int ptr_align)
         if (g_table[i].m == m && g_table[i].n == n && g_table[i].k == k && resolved[i] >= 0 &&
             config_supports(resolved[i], m, n, k, ptr_align))
             return {resolved[i], g_table[i].group_m, g_table[i].ksplit > 0 ? g_table[i].ksplit : 1, g_table[i].spread};
-    return heuristic(m, n, k, ptr_align);
+    return heuristic(m, n, k, ptr_align, has_ws);
 }
 
 // The scaled output has fewer kernels to choose from: the table's choice when that
 // configuration has the output form, else the best pipelined one that has it, else what the
 // heuristic says for skinny shapes, else the generic kernel.
-static Choice select_scaled(int m, int n, int k, int ptr_align)
+static Choice select_scaled(int m, int n, int k, int ptr_align, bool has_ws)
 {
-    const Choice ch = select_config(m, n, k, ptr_align);
+    const Choice ch = select_config(m, n, k, ptr_align, has_ws);
     if (ch.ksplit <= 1 && scaled_launcher(ch.cfg)) return ch;
+    // K split: the int32 kernel of any pipelined configuration leaves partial sums in the
+    // workspace, and the kernel that adds them up scales and rounds
+    if (ch.ksplit > 1 && has_ws && g_configs[ch.cfg].kind == KIND_TILE16) return ch;
     if (fast_path_ok(m, n, k, ptr_align) && k % 128 == 0) {
         int best = -1;
         double best_cost = 1e300;
@@ -473,7 +572,7 @@ static Choice select_scaled(int m, int n, int k, int ptr_align)
         }
         if (best >= 0) return {best, 4, 1};
     }
-    const Choice h = heuristic(m, n, k, ptr_align);
+    const Choice h = heuristic(m, n, k, ptr_align, false);
     if (h.ksplit <= 1 && scaled_launcher(h.cfg)) return h;
     return {0, 1, 1};
 }
@@ -504,11 +603,78 @@ static int fail_launch(hipError_t e)
     return QM_ERR_LAUNCH;
 }
 
+// The splits of K that have work (with kps K-steps per split only ceil(kt / kps) have any)
+// and the workspace they fill: one padded tile of int32 per (split, tile).
+static int effective_ksplit(const ConfigDesc &d, int k, int ksplit)
+{
+    if (d.kind != KIND_TILE16 || ksplit <= 1) return 1;
+    const int kt = k / d.bk, kps = (kt + ksplit - 1) / ksplit;
+    return (kt + kps - 1) / kps;
+}
+
+static size_t split_workspace_bytes(const ConfigDesc &d, int m, int n, int ksplit)
+{
+    const size_t tiles = (size_t)((m + d.bm - 1) / d.bm) * (size_t)((n + d.bn - 1) / d.bn);
+    return tiles * (size_t)ksplit * (size_t)d.bm * (size_t)d.bn * sizeof(int32_t);
+}
+
+static bool workspace_fits(const ConfigDesc &d, int m, int n, int ksplit, const void *ws, size_t ws_bytes)
+{
+    return ws != nullptr && ((uintptr_t)ws & 15) == 0 && ws_bytes >= split_workspace_bytes(d, m, n, ksplit);
+}
+
+static Choice choice_from_code(int cfg)
+{
+    Choice ch;
+    ch.cfg = cfg & 0xFFFF;
+    ch.group_m = (cfg >> 16) & 0xFF;
+    ch.ksplit = (cfg >> 24) & 0x3F;
+    ch.spread = (cfg >> 30) & 1;
+    if (ch.group_m == 0) ch.group_m = 4;
+    if (ch.ksplit == 0) ch.ksplit = 1;
+    return ch;
+}
+
+// GEMM with K split into ch.ksplit (> 1, normalised) through the workspace, then the sum of
+// the splits into C in the output form p.out.
+static hipError_t launch_split_with_workspace(GemmArgs p, const Choice &ch, void *ws, hipStream_t s)
+{
+    const ConfigDesc &d = g_configs[ch.cfg];
+    SplitReduceArgs q;
+    q.ws = static_cast<const v4i *>(ws);
+    q.C = p.C;
+    q.M = p.M;
+    q.N = p.N;
+    q.tiles_m = (p.M + d.bm - 1) / d.bm;
+    q.tiles_n = (p.N + d.bn - 1) / d.bn;
+    q.group_m = ch.group_m < 1 ? 1 : (ch.group_m > q.tiles_m ? q.tiles_m : ch.group_m);  // as the launcher clamps it
+    q.ksplit = ch.ksplit;
+    q.BM = d.bm;
+    q.BN = d.bn;
+    q.WGN = d.wgn;
+    q.FM = d.bm / d.wgm / 16;
+    q.FN = d.bn / d.wgn / 16;
+    q.waves = d.waves;
+    q.row_scale = p.row_scale;
+    q.col_scale = p.col_scale;
+    q.out = p.out;
+    p.out = OUT_I32;
+    p.row_scale = p.col_scale = nullptr;
+    p.ws = static_cast<int32_t *>(ws);
+    hipError_t e = d.launch(p, s, ch.group_m | (ch.ksplit << 8) | (ch.spread << 16));
+    if (e != hipSuccess) return e;
+    const size_t pieces = (size_t)q.tiles_m * q.tiles_n * (size_t)(d.bm * d.bn / 4);
+    if (pieces > 0x7fffff00ULL) return hipErrorInvalidValue;
+    splitk_reduce_kernel<<<dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, s>>>(q);
+    return hipGetLastError();
+}
+
 }  // namespace qm
 
 using namespace qm;
 
-QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg)
+QM_EXPORT int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg,
+                            void *workspace, size_t workspace_bytes)
 {
     const int st = check_gemm_args(A, B, C, m, n, k);
     if (st != QM_OK) return st;
@@ -521,22 +687,23 @@ QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n
         return e == hipSuccess ? QM_OK : fail_launch(e);
     }
     const int align = ptr_alignment(A, B);
+    const bool has_ws = workspace != nullptr && workspace_bytes > 0;
     Choice ch;
     if (cfg == QM_CFG_AUTO) {
-        ch = select_config(m, n, k, align);
+        ch = select_config(m, n, k, align, has_ws);
     } else {
-        ch.cfg = cfg & 0xFFFF;
-        ch.group_m = (cfg >> 16) & 0xFF;
-        ch.ksplit = (cfg >> 24) & 0x3F;
-        ch.spread = (cfg >> 30) & 1;
-        if (ch.group_m == 0) ch.group_m = 4;
-        if (ch.ksplit == 0) ch.ksplit = 1;
+        ch = choice_from_code(cfg);
         if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
         if (ch.ksplit > 1 && g_configs[ch.cfg].kind != KIND_TILE16) return QM_ERR_CONFIG;
     }
+    ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
     const GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(C), m, n, k};
+    if (ch.ksplit > 1 && workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) {
+        const hipError_t e = launch_split_with_workspace(p, ch, workspace, s);
+        return e == hipSuccess ? QM_OK : fail_launch(e);
+    }
     if (ch.ksplit > 1) {
-        // split-K partial sums meet in C by integer atomic adds: C starts from zero
+        // no workspace: split-K partial sums meet in C by integer atomic adds, C starts from zero
         const size_t cnt = (size_t)m * (size_t)n;
         fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(C), cnt);
         const hipError_t ez = hipGetLastError();
@@ -546,8 +713,14 @@ QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n
     return e == hipSuccess ? QM_OK : fail_launch(e);
 }
 
-QM_EXPORT int qm_gemm_i4_scaled_cfg(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
-                                    const float *col_scale, int out_dtype, void *stream, int cfg)
+QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg)
+{
+    return qm_gemm_i4_ws(A, B, C, m, n, k, stream, cfg, nullptr, 0);
+}
+
+QM_EXPORT int qm_gemm_i4_scaled_ws(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
+                                   const float *col_scale, int out_dtype, void *stream, int cfg, void *workspace,
+                                   size_t workspace_bytes)
 {
     if (out_dtype != QM_OUT_F16 && out_dtype != QM_OUT_BF16) return QM_ERR_DTYPE;
     if (m < 0 || n < 0 || k < 0 || (k & 1)) return QM_ERR_SHAPE;
@@ -563,32 +736,61 @@ QM_EXPORT int qm_gemm_i4_scaled_cfg(const void *A, const void *B, void *D, int m
         return e == hipSuccess ? QM_OK : fail_launch(e);
     }
     const int align = ptr_alignment(A, B);
-    Choice ch;
-    if (cfg == QM_CFG_AUTO) {
-        ch = select_scaled(m, n, k, align);
-    } else {
-        ch.cfg = cfg & 0xFFFF;
-        ch.group_m = (cfg >> 16) & 0xFF;
-        ch.ksplit = 1;
-        ch.spread = (cfg >> 30) & 1;
-        if (ch.group_m == 0) ch.group_m = 4;
-        if (((cfg >> 24) & 0x3F) > 1) return QM_ERR_CONFIG;  // partial sums cannot meet in a rounded output
-        if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
-    }
-    const LaunchFn launch = scaled_launcher(ch.cfg);
-    if (!launch) return QM_ERR_CONFIG;
+    const bool has_ws = workspace != nullptr && workspace_bytes > 0;
     GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(D), m, n, k};
     p.row_scale = row_scale;
     p.col_scale = col_scale;
     p.out = out_dtype == QM_OUT_F16 ? OUT_F16 : OUT_BF16;
+    Choice ch;
+    if (cfg == QM_CFG_AUTO) {
+        ch = select_scaled(m, n, k, align, has_ws);
+        ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
+        if (ch.ksplit > 1 && !workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) {
+            ch = select_scaled(m, n, k, align, false);  // too small a workspace: as without one
+            ch.ksplit = 1;
+        }
+    } else {
+        ch = choice_from_code(cfg);
+        if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
+        if (ch.ksplit > 1 && g_configs[ch.cfg].kind != KIND_TILE16) return QM_ERR_CONFIG;
+        ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
+        // partial sums cannot meet in a rounded output: a K split needs the workspace
+        if (ch.ksplit > 1 && !workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) return QM_ERR_CONFIG;
+    }
+    if (ch.ksplit > 1) {
+        const hipError_t e = launch_split_with_workspace(p, ch, workspace, s);
+        return e == hipSuccess ? QM_OK : fail_launch(e);
+    }
+    const LaunchFn launch = scaled_launcher(ch.cfg);
+    if (!launch) return QM_ERR_CONFIG;
     const hipError_t e = launch(p, s, ch.group_m | (1 << 8) | (ch.spread << 16));
     return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
+QM_EXPORT int qm_gemm_i4_scaled_cfg(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
+                                    const float *col_scale, int out_dtype, void *stream, int cfg)
+{
+    return qm_gemm_i4_scaled_ws(A, B, D, m, n, k, row_scale, col_scale, out_dtype, stream, cfg, nullptr, 0);
 }
 
 QM_EXPORT int qm_gemm_i4_scaled(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
                                 const float *col_scale, int out_dtype, void *stream)
 {
-    return qm_gemm_i4_scaled_cfg(A, B, D, m, n, k, row_scale, col_scale, out_dtype, stream, QM_CFG_AUTO);
+    return qm_gemm_i4_scaled_ws(A, B, D, m, n, k, row_scale, col_scale, out_dtype, stream, QM_CFG_AUTO, nullptr, 0);
+}
+
+QM_EXPORT size_t qm_gemm_workspace_bytes(int m, int n, int k, int ptr_align, int cfg, int scaled)
+{
+    if (m < 1 || n < 1 || k < 2 || (k & 1)) return 0;
+    Choice ch;
+    if (cfg == QM_CFG_AUTO) {
+        ch = scaled ? select_scaled(m, n, k, ptr_align, true) : select_config(m, n, k, ptr_align, true);
+    } else {
+        ch = choice_from_code(cfg);
+        if (!config_supports(ch.cfg, m, n, k, ptr_align)) return 0;
+    }
+    const int ks = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
+    return ks > 1 ? split_workspace_bytes(g_configs[ch.cfg], m, n, ks) : 0;
 }
 
 QM_EXPORT int qm_config_has_scaled(int cfg)
@@ -605,7 +807,7 @@ QM_EXPORT int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, in
 QM_EXPORT int qm_select_config(int m, int n, int k, int ptr_align)
 {
     if (m < 1 || n < 1 || k < 2 || (k & 1)) return QM_ERR_SHAPE;
-    const Choice ch = select_config(m, n, k, ptr_align);
+    const Choice ch = select_config(m, n, k, ptr_align, true);
     return ch.cfg | (ch.group_m << 16) | (ch.ksplit << 24) | (ch.spread << 30);
 }
 

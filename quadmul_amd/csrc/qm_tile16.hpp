@@ -360,6 +360,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // treat them as general values and copy them around.
     int c_item = blockIdx.x, c_kt = 0, c_m0, c_n0, c_kt0, c_KT;  // the item being contracted
     char *tile_c = nullptr;  // its corner in C (wave-uniform)
+    v4i *split_ws = nullptr;  // this lane's place in the item's workspace slot (K split with a workspace)
     // scaled output: this lane's scales for the item, as the MFMA leaves a block (row r of
     // every block row, columns 4g..4g+3 of every block column)
     typedef float v4f __attribute__((ext_vector_type(4)));
@@ -444,6 +445,14 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     auto write_guarded = [&](auto ib_, auto j_) __attribute__((always_inline)) {
         constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value;
         const v4i v = take_block(ib_, j_);
+        if constexpr (OUT == OUT_I32) {
+            if (split_ws != nullptr) {
+                // K-split partial sums with a workspace: the block as it is, 16 bytes per lane
+                // (whole 1 KiB lines per wave; the padding of a ragged tile has room there)
+                split_ws[(ib * FN + j) * 64] = v;
+                return;
+            }
+        }
         const int m = (c_m0 + ib * 16) + (wm * Cfg::WM + r), n = (c_n0 + j * 16) + (wn * Cfg::WN + g * 4);
         if constexpr (OUT != OUT_I32) {
             if (m < p.M) {
@@ -463,6 +472,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             if (ksplit > 1) {
                 // every partial accumulator is a multiple of 256, so the shifted partials add
                 // up to the shifted total; integer atomics make the order irrelevant
+                // (this branch only runs without a workspace: see below)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -593,6 +603,12 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         uint32_t bmask = c_kt + 1 < c_KT ? amask : 0u;
         asm volatile("" : "+s"(bmask));
         tile_c = reinterpret_cast<char *>(p.C) + ((size_t)c_m0 * p.N + c_n0) * ESZ;
+        if constexpr (OUT == OUT_I32 && !whole) {
+            // workspace slot of a K-split item: (split, tile) in the order locate() numbers them
+            if (p.ws != nullptr && ksplit > 1)
+                split_ws = reinterpret_cast<v4i *>(p.ws) +
+                           ((size_t)xcd_contiguous_id(c_item, nitems) * WAVES + wave) * (FM * FN * 64) + lane;
+        }
         k_step(bmask, std::integral_constant<int, 0>{}, std::false_type{});
         k_step(amask, std::integral_constant<int, 1>{}, std::integral_constant<bool, whole>{});
         // Let the last MFMAs retire before their accumulators are read (the compiler does not

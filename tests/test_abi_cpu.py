@@ -87,12 +87,35 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_quantize_pack_i4(one, 1, one, None, 4, 8, None) == -1
     assert lib.qm_quantize_pack_i4(ctypes.c_void_p(4097), 1, one, one, 4, 8, None) == -5
     assert lib.qm_quantize_pack_i4(None, 3, None, None, 0, 8, None) == 0
+    # the forms with a workspace: same checks; the workspace itself is optional
+    assert lib.qm_gemm_i4_ws(one, one, one, 4, 4, 3, None, -1, None, 0) == -2
+    assert lib.qm_gemm_i4_ws(one, one, None, 4, 4, 4, None, -1, one, 1 << 20) == -1
+    assert lib.qm_gemm_i4_ws(None, None, None, 0, 4, 4, None, -1, None, 0) == 0
+    assert lib.qm_gemm_i4_ws(one, one, one, 64, 64, 512, None, qm.config_id("t64x64x128_w2x2_m0") | (2 << 24), one, 1 << 20) == -3
+    assert lib.qm_gemm_i4_scaled_ws(one, one, one, 4, 4, 4, None, None, 7, None, -1, None, 0) == -6
+    assert lib.qm_gemm_i4_scaled_ws(one, one, one, 256, 256, 512, None, None, 1, None, qm.config_id("q256x256_w2x2_s4o1") | (2 << 24), one, 4096) == -3
     has = [qm.config_has_scaled(i) for i in range(qm.num_configs())]
     assert has[qm.config_id("generic")] and has[qm.config_id("q256x256_w2x2_s4o1")] and has[qm.config_id("s1x1_w8_u4")]
     assert not has[qm.config_id("t64x64x128_w2x2_m0")] and not has[qm.config_id("q256x128_w2x2_s3o2")]
     for code in (0, -1, -2, -3, -4, -5, -6):
         assert lib.qm_status_string(code)
     assert b"gfx950" in lib.qm_version()
+
+
+def test_workspace_sizes():
+    q128 = qm.config_id("q128x128_w2x2_s4o1")
+    # one padded int32 tile per (split, tile): 2 x 3 tiles of 128 x 128, 4 splits
+    assert qm.workspace_bytes(200, 300, 4096, q128 | (4 << 24)) == 4 * 6 * 128 * 128 * 4
+    # splits without work do not count: 3 K-steps cannot feed 8 splits
+    assert qm.workspace_bytes(200, 300, 384, q128 | (8 << 24)) == 3 * 6 * 128 * 128 * 4
+    assert qm.workspace_bytes(200, 300, 4096, q128) == 0                       # no split asked for
+    assert qm.workspace_bytes(200, 300, 4096, qm.config_id("t128x128x128_w2x2_m0") | (4 << 24)) == 0
+    assert qm.workspace_bytes(8192, 8192, 8192) == 0                           # plenty of tiles
+    code = qm.select_config(128, 8192, 28672)
+    assert (code >> 24) & 0x3F > 1
+    assert qm.workspace_bytes(128, 8192, 28672) == qm.workspace_bytes(128, 8192, 28672, code) > 0
+    assert qm.workspace_bytes(128, 8192, 28672, scaled=True) > 0
+    assert qm.workspace_bytes(0, 8192, 28672) == 0 and qm.workspace_bytes(128, 8192, 3) == 0
 
 
 def test_config_registry():

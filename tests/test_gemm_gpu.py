@@ -5,17 +5,17 @@ import pytest
 import torch
 
 import quadmul_amd as qm
-from util import SEED_BASE, make_operands, pack_cpu, poisoned_c
+from util import C_POISON, SEED_BASE, make_operands, pack_cpu, poisoned_c
 
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
 
 
-def run_gemm(ap, bp, m, n, k, cfg=qm.CFG_AUTO):
+def run_gemm(ap, bp, m, n, k, cfg=qm.CFG_AUTO, workspace=True):
     a_d, b_d = ap.to(DEV), bp.to(DEV)
     c_d = poisoned_c(m, n, DEV)
-    qm.gemm_cfg(a_d, b_d, c_d, m, n, k, cfg)
+    qm.gemm_cfg(a_d, b_d, c_d, m, n, k, cfg, workspace)
     torch.cuda.synchronize()
     return c_d.cpu().numpy()
 
@@ -50,9 +50,13 @@ def test_every_config_matches_oracle(oracle_mod, shape):
         # 8 leaves some splits empty on short K)
         variants = [(1, 1), (3, 1)] + ([(2, 2), (1, 3), (4, 8)] if name.startswith("q") else [])
         for gm, ks in variants:
-            got = run_gemm(ap, bp, m, n, k, cfg | (gm << 16) | (ks << 24))
-            bad = oracle_mod.compare(got, want)
-            assert bad == -1, f"{name} group_m={gm} ksplit={ks}: first mismatch at flat index {bad}: got {got.flat[bad]} want {want.flat[bad]}"
+            # a K split with a workspace (partial tiles, then a kernel that adds them up) and
+            # without one (atomic adds into a zero-filled C)
+            for ws in ([True, None] if ks > 1 else [True]):
+                got = run_gemm(ap, bp, m, n, k, cfg | (gm << 16) | (ks << 24), ws)
+                bad = oracle_mod.compare(got, want)
+                assert bad == -1, (f"{name} group_m={gm} ksplit={ks} workspace={ws}: first mismatch at flat index {bad}: "
+                                   f"got {got.flat[bad]} want {want.flat[bad]}")
         ran += 1
     assert ran >= 2
     got = run_gemm(ap, bp, m, n, k)
@@ -121,8 +125,9 @@ def test_extremes_closed_form_on_every_config(shape):
             continue
         assert (run_gemm(lo_a, lo_b, m, n, k, cfg) == 64 * k).all(), name   # largest positive accumulator
         assert (run_gemm(lo_a, hi_b, m, n, k, cfg) == -56 * k).all(), name  # most negative accumulator
-        if name.startswith("q"):  # split K: partial sums meet by atomic adds
+        if name.startswith("q"):  # split K: partial sums meet in a workspace, or by atomic adds
             assert (run_gemm(lo_a, hi_b, m, n, k, cfg | (4 << 24)) == -56 * k).all(), name
+            assert (run_gemm(lo_a, hi_b, m, n, k, cfg | (4 << 24), None) == -56 * k).all(), name
 
 
 def test_largest_exact_k_and_beyond(oracle_mod):
@@ -323,3 +328,69 @@ def test_large_configs(oracle_mod, row):
     colsum = a.to(torch.int64).sum(0)
     want_cs = (b.to(torch.int64) * colsum).sum(1)
     assert torch.equal(got_d.to(torch.int64).sum(0).cpu(), want_cs)
+
+
+@pytest.mark.parametrize("shape", [(128, 1024, 14336), (200, 300, 2048), (257, 511, 1280), (70, 4100, 4096)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_split_k_workspace_forms(oracle_mod, shape):
+    """K split on the pipelined kernel: the caller's workspace in every form it can take --
+    allocated by the wrapper, the caller's own tensor (exact size, larger, holding garbage),
+    too small or absent (then atomics) -- gives the oracle's result."""
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 5200 + m)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    ran = 0
+    for cfg, name in enumerate(qm.config_names()):
+        if not name.startswith("q") or not qm.config_supports(cfg, m, n, k):
+            continue
+        for gm, ks in [(1, 2), (3, 5), (8, 8)]:
+            code = cfg | (gm << 16) | (ks << 24)
+            need = qm.workspace_bytes(m, n, k, code)
+            assert need > 0 and need % 16 == 0
+            garbage = torch.randint(-128, 128, (need + 4096,), dtype=torch.int8, device=DEV).view(torch.uint8)
+            for what, ws in [("wrapper", True), ("exact", garbage[:need]), ("larger", garbage), ("too small", garbage[:need - 16]),
+                             ("none", None)]:
+                c_d = poisoned_c(m, n, DEV)
+                qm.gemm_cfg(a_d, b_d, c_d, m, n, k, code, ws)
+                torch.cuda.synchronize()
+                bad = oracle_mod.compare(c_d.cpu().numpy(), want)
+                assert bad == -1, f"{name} group_m={gm} ksplit={ks} workspace {what}: first mismatch at flat index {bad}"
+        ran += 1
+    assert ran >= 4
+
+
+def test_auto_choice_splits_k_and_matches(oracle_mod):
+    # few tiles, long K: the automatic choice splits K; extension module and wrapper agree with the oracle
+    import quadmul
+
+    m, n, k = 128, 2048, 28672
+    code = qm.select_config(m, n, k)
+    assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
+    assert qm.workspace_bytes(m, n, k) > 0
+    a, b = make_operands(m, n, k, SEED_BASE + 5300)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    for fn in (lambda c: quadmul.gemm(a_d, b_d, c, m, n, k), lambda c: qm.gemm(a_d, b_d, c, m, n, k),
+               lambda c: qm.gemm(a_d, b_d, c, m, n, k, workspace=None), lambda c: torch.ops.quadmul.gemm(a_d, b_d, c, m, n, k)):
+        c_d = poisoned_c(m, n, DEV)
+        fn(c_d)
+        torch.cuda.synchronize()
+        assert oracle_mod.compare(c_d.cpu().numpy(), want) == -1
+    # captured in a graph (the workspace comes from the allocator's graph pool) and replayed
+    c_d = poisoned_c(m, n, DEV)
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        quadmul.gemm(a_d, b_d, c_d, m, n, k)
+        with torch.cuda.graph(g, stream=side):
+            quadmul.gemm(a_d, b_d, c_d, m, n, k)
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        c_d.fill_(C_POISON)
+        g.replay()
+        torch.cuda.synchronize()
+        assert oracle_mod.compare(c_d.cpu().numpy(), want) == -1

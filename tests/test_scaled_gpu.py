@@ -83,14 +83,19 @@ def test_missing_scales_and_k_zero(oracle_mod):
 
 
 def test_rejections():
-    m, n, k = 64, 64, 128
+    m, n, k = 64, 64, 512
     a = torch.zeros((m, k // 2), dtype=torch.int8, device=DEV)
     d = torch.zeros((m, n), dtype=torch.float16, device=DEV)
     names = qm.config_names()
     with pytest.raises(qm.QuadmulError):  # a plain tile kernel has no scaled output
         qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("t64x64x128_w2x2_m0"))
-    with pytest.raises(qm.QuadmulError):  # partial sums cannot meet in a rounded output
-        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s4o1") | (2 << 24))
+    with pytest.raises(qm.QuadmulError):  # partial sums cannot meet in a rounded output: a K split needs a workspace
+        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s4o1") | (2 << 24), workspace=None)
+    with pytest.raises(qm.QuadmulError):
+        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s4o1") | (2 << 24),
+                       workspace=torch.empty(1024, dtype=torch.uint8, device=DEV))
+    with pytest.raises(qm.QuadmulError):  # only the pipelined kernel splits K
+        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("s4x1_w8_u2") | (2 << 24))
     with pytest.raises(qm.QuadmulError):
         qm.gemm_scaled(a, a, torch.zeros((m, n), dtype=torch.int32, device=DEV), m, n, k)
     with pytest.raises(qm.QuadmulError):
@@ -166,3 +171,37 @@ def test_extension_module_and_dispatcher_op(oracle_mod):
             assert (bits(d4) == want).all()
     with pytest.raises(RuntimeError):
         quadmul.gemm_scaled(a_d, b_d, torch.zeros((m, n), dtype=torch.float32, device=DEV), m, n, k)
+
+
+@pytest.mark.parametrize("shape", [(128, 1024, 14336), (200, 300, 2048), (257, 511, 1280)], ids=lambda s: "x".join(map(str, s)))
+def test_scaled_with_k_split_through_a_workspace(oracle_mod, shape):
+    """With a workspace the scaled form takes K splits on every pipelined configuration: the
+    int32 partial tiles are added up, scaled and rounded by the second kernel."""
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 7300 + m)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    rs, cs = make_scales(m, n, SEED_BASE + 7400 + m)
+    c = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    a_d, b_d, rs_d, cs_d = ap.to(DEV), bp.to(DEV), rs.to(DEV), cs.to(DEV)
+    ran = 0
+    for dtype, out in DTYPES:
+        want = oracle_mod.scale_round16(c, rs.numpy(), cs.numpy(), out)
+        want_rows_only = oracle_mod.scale_round16(c, rs.numpy(), None, out)
+        for cfg, name in enumerate(qm.config_names()):
+            if not name.startswith("q") or not qm.config_supports(cfg, m, n, k):
+                continue
+            for gm, ks in [(1, 2), (3, 5)]:
+                code = cfg | (gm << 16) | (ks << 24)
+                assert qm.workspace_bytes(m, n, k, code, scaled=True) > 0
+                d = poisoned_d(m, n, dtype)
+                qm.gemm_scaled(a_d, b_d, d, m, n, k, rs_d, cs_d, code)
+                torch.cuda.synchronize()
+                got = bits(d)
+                bad = np.flatnonzero(got != want)
+                assert bad.size == 0, f"{name} {dtype} group_m={gm} ksplit={ks}: {bad.size} mismatches, first at {bad[0]}"
+            d = poisoned_d(m, n, dtype)
+            qm.gemm_scaled(a_d, b_d, d, m, n, k, rs_d, None, cfg | (4 << 24))
+            torch.cuda.synchronize()
+            assert (bits(d) == want_rows_only).all(), name
+            ran += 1
+    assert ran >= 8
