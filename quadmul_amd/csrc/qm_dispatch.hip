@@ -2,7 +2,9 @@
 // choice and launches.  Takes the place of the reference's host side:
 // wrapper (kernel.cu:334-385), LAUNCH_KERNEL_IF_CONDITION (kernel.cu:321-332)
 // and launch_igemm (kernel.cu:268-289).
+#include <algorithm>
 #include <atomic>
+#include <cmath>
 #include <cstring>
 #include <mutex>
 
@@ -383,6 +385,8 @@ static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
 }
 #define QM_SKINNY(FM, FN, NW, U) \
     hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U>>(p, s, gm); }
+#define QM_SKINNYP(FM, FN, NW, U) \
+    hipError_t QM_SKINNYP_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U, 1>>(p, s, gm); }
 #include "qm_configs.inc"
 
 // --------------------------------------------------------------------------
@@ -412,6 +416,9 @@ static const ConfigDesc g_configs[] = {
 #define QM_SKINNY(FM, FN, NW, U)                                                     \
     {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
      &QM_SKINNY_FN(FM, FN, NW, U)},
+#define QM_SKINNYP(FM, FN, NW, U)                                                     \
+    {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U) "p", KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
+     &QM_SKINNYP_FN(FM, FN, NW, U)},
 #include "qm_configs.inc"
 };
 static constexpr int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
@@ -488,16 +495,20 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
     if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
     if (m <= 64) {
         const int fm = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
-        const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w8_u2");
+        const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w8_u4p");
         const int id = find_config(name);
         if (id >= 0) return {id, 1, 1};
     }
     // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency),
     // over the configurations that can run this K.  Efficiencies are measured ratios.
-    static const struct { const char *name; double eff; } cands[] = {
-        {"q256x256_w2x2_s4o1", 1.00}, {"q256x128_w2x2_s4o1", 0.82}, {"q128x256_w2x2_s4o1", 0.82}, {"q128x128_w2x2_s4o1", 0.66},
-        {"t256x256x128_w4x2_m0", 0.78}, {"t128x128x128_w2x2_m0", 0.60}, {"t64x128x128_w2x2_m0", 0.40},
-        {"t128x64x128_w2x2_m0", 0.40},  {"t64x64x128_w2x2_m0", 0.30},
+    // eff: throughput per tile area relative to the 256 x 256 pipelined kernel with the GPU
+    // full.  share: the plain tile kernels run several small workgroups per CU, and one
+    // alone does not run that many times faster -- a launch with fewer tiles per CU than
+    // this is priced as if it had this many.
+    static const struct { const char *name; double eff, share; } cands[] = {
+        {"q256x256_w2x2_s4o1", 1.00, 1.0}, {"q256x128_w2x2_s4o1", 0.82, 1.0}, {"q128x256_w2x2_s4o1", 0.82, 1.0},
+        {"q128x128_w2x2_s4o1", 0.60, 1.0}, {"t256x256x128_w4x2_m0", 0.70, 1.0}, {"t128x128x128_w2x2_m0", 0.35, 1.0},
+        {"t64x128x128_w2x2_m0", 0.27, 1.5}, {"t128x64x128_w2x2_m0", 0.27, 1.5}, {"t64x64x128_w2x2_m0", 0.28, 2.0},
     };
     int best = 0, best_ks = 1;
     double best_cost = 1e300;
@@ -512,12 +523,13 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         // enough that splitting only pays when each split keeps a long K of its own
         // (measured: wins at K = 28672, loses at K = 8192).
         // Cost in units of 16.5 ps (one K-step of the 256 x 256 tile = 65536): K-steps per
-        // item x tile area / efficiency, plus 3 us per round of workgroups for filling the
+        // item x tile area / efficiency, plus 4 us per round of workgroups (2 us for the plain tile kernels) for filling the
         // ring and writing out, plus the split's own cost.
         const int kt = (k + 127) / 128;
         auto cost_of = [&](int ks_) {
-            const long long rounds = (tiles * ks_ + 255) / 256;
-            return (double)rounds * ((double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + 180000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
+            double rounds = (double)((tiles * ks_ + 255) / 256);
+            if (d.kind == KIND_TILE) rounds = std::max((double)tiles / 256.0, c.share);
+            return rounds * (double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + (d.kind == KIND_TILE ? 120000.0 : std::ceil(rounds) * 240000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
         };
         int ks = 1;
         double cost = cost_of(1);
@@ -529,6 +541,14 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
             if (ks > 1) cost = (double)d.bm * d.bn / c.eff * ((kt + ks - 1) / ks) * 1.25 + 180000.0;
         }
         if (cost < best_cost) { best_cost = cost; best = id; best_ks = ks; }
+    }
+    if (m <= 128) {
+        // 65..128 rows: the wave-level split-K kernel with eight row blocks has no ring to
+        // fill and no second kernel, and wins while N x K is small (measured: about 2 us
+        // plus 0.38 us per million elements of B, in the units above)
+        const int id = find_config("s8x1_w8_u1");
+        const double cost_s = (2.0 + (double)n * (double)k / 2.6e6) / 1.65e-5;
+        if (id >= 0 && cost_s < best_cost) return {id, 1, 1};
     }
     const int ksplit = best_ks;
     return {best, 4, ksplit};
