@@ -2,7 +2,7 @@
 //
 // The reference has no such path: its smallest tile is 32 rows (configs.cu) and
 // shapes outside its table are skipped (kernel.cu:340-385).  Here a workgroup
-// owns 16*FN rows of B (columns of C) and all of M (padded to 16*FM <= 64); its
+// owns 16*FN rows of B (columns of C) and all of M (padded to 16*FM <= 128); its
 // NW waves split K between them in 128-nibble chunks, each wave streaming its
 // share of B straight from HBM into registers, and the partial 16x16 blocks are
 // summed through LDS.  One launch, no workspace, no atomics, C overwritten.
