@@ -394,3 +394,37 @@ def test_auto_choice_splits_k_and_matches(oracle_mod):
         g.replay()
         torch.cuda.synchronize()
         assert oracle_mod.compare(c_d.cpu().numpy(), want) == -1
+
+
+def test_random_shapes_through_the_automatic_choice():
+    """A seeded sweep of shapes nobody tuned for, through qm_gemm_i4's own choice of kernel
+    (table, cost model, K split with a workspace, generic fallback), against an fp32 matmul
+    on the GPU (exact: every partial sum is an integer below 2^24)."""
+    import quadmul
+
+    rng = np.random.default_rng(SEED_BASE + 5400)
+    seen = set()
+    for i in range(160):
+        m = int(np.exp(rng.uniform(0, np.log(1500)))) if i % 3 else int(rng.integers(1, 140))
+        n = int(np.exp(rng.uniform(0, np.log(6000))))
+        kind = i % 4
+        k = int(np.exp(rng.uniform(np.log(2), np.log(12000))))
+        k = max(2, [k // 128 * 128, k // 32 * 32, k // 2 * 2, k // 128 * 128][kind])
+        if i % 10 == 0:
+            m, k = int(rng.integers(65, 129)), int(rng.integers(8, 64)) * 128   # the 128-row skinny kernel
+        if i % 10 == 5:   # few tiles, long K: the pipelined kernel with K split through a workspace
+            m, n, k = int(rng.integers(129, 600)), int(rng.integers(256, 1024)), int(rng.integers(64, 94)) * 128
+        if i % 10 == 7:   # many tiles: the pipelined kernel, persistent grid
+            m, n, k = int(rng.integers(700, 1500)), int(rng.integers(3000, 6000)), int(rng.integers(4, 16)) * 128
+        a = torch.randint(-8, 8, (m, k), dtype=torch.int8, generator=torch.Generator().manual_seed(1000 + i))
+        b = torch.randint(-8, 8, (n, k), dtype=torch.int8, generator=torch.Generator().manual_seed(2000 + i))
+        a_d, b_d = pack_cpu(a).to(DEV), pack_cpu(b).to(DEV)
+        want = fp32_matmul_on_gpu(a, b)
+        c_d = poisoned_c(m, n, DEV)
+        quadmul.gemm(a_d, b_d, c_d, m, n, k)
+        torch.cuda.synchronize()
+        code = qm.select_config(m, n, k)
+        name = qm.config_name(code & 0xFFFF)
+        seen.add(name[0] + ("+split" if (code >> 24) & 0x3F > 1 else ""))
+        assert torch.equal(c_d, want), f"{m}x{n}x{k} ({name}, ksplit {(code >> 24) & 0x3F})"
+    assert {"g", "s", "t", "q", "q+split"} <= seen, seen

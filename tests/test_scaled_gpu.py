@@ -205,3 +205,27 @@ def test_scaled_with_k_split_through_a_workspace(oracle_mod, shape):
             assert (bits(d) == want_rows_only).all(), name
             ran += 1
     assert ran >= 8
+
+
+def test_scaled_random_shapes_through_the_automatic_choice():
+    """The same sweep for the scaled output, against torch's float32 arithmetic on the exact
+    int32 product (two separate float32 multiplications, then torch's rounding to 16 bits)."""
+    rng = np.random.default_rng(SEED_BASE + 7500)
+    for i in range(80):
+        m = int(np.exp(rng.uniform(0, np.log(1200)))) if i % 3 else int(rng.integers(1, 140))
+        n = int(np.exp(rng.uniform(0, np.log(5000))))
+        k = int(np.exp(rng.uniform(np.log(2), np.log(12000))))
+        k = max(2, [k // 128 * 128, k // 32 * 32, k // 2 * 2, k // 128 * 128][i % 4])
+        if i % 8 == 0:
+            m, k = int(rng.integers(65, 129)), int(rng.integers(16, 96)) * 128
+        a = torch.randint(-8, 8, (m, k), dtype=torch.int8, generator=torch.Generator().manual_seed(3000 + i))
+        b = torch.randint(-8, 8, (n, k), dtype=torch.int8, generator=torch.Generator().manual_seed(4000 + i))
+        rs, cs = make_scales(m, n, 5000 + i)
+        a_d, b_d, rs_d, cs_d = pack_cpu(a).to(DEV), pack_cpu(b).to(DEV), rs.to(DEV), cs.to(DEV)
+        c32 = (a.to(DEV).float() @ b.to(DEV).float().t())   # exact integers in fp32
+        dtype = torch.float16 if i % 2 else torch.bfloat16
+        want = ((c32 * rs_d[:, None]) * cs_d[None, :]).to(dtype)
+        d = poisoned_d(m, n, dtype)
+        qm.gemm_scaled(a_d, b_d, d, m, n, k, rs_d, cs_d)
+        torch.cuda.synchronize()
+        assert torch.equal(d.view(torch.int16), want.view(torch.int16)), f"{m}x{n}x{k} {dtype}"
