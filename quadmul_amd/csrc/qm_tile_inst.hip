@@ -114,6 +114,10 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK_9(...)
 #define QM_PICK_10(...)
 #define QM_PICK_11(...)
+#define QM_PICK_12(...)
+#define QM_PICK_13(...)
+#define QM_PICK_14(...)
+#define QM_PICK_15(...)
 #define QM_PICK16_0(...)
 #define QM_PICK16_1(...)
 #define QM_PICK16_2(...)
@@ -126,6 +130,10 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16_9(...)
 #define QM_PICK16_10(...)
 #define QM_PICK16_11(...)
+#define QM_PICK16_12(...)
+#define QM_PICK16_13(...)
+#define QM_PICK16_14(...)
+#define QM_PICK16_15(...)
 #define QM_PICK16S_0(...)
 #define QM_PICK16S_1(...)
 #define QM_PICK16S_2(...)
@@ -138,6 +146,10 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16S_9(...)
 #define QM_PICK16S_10(...)
 #define QM_PICK16S_11(...)
+#define QM_PICK16S_12(...)
+#define QM_PICK16S_13(...)
+#define QM_PICK16S_14(...)
+#define QM_PICK16S_15(...)
 #if QM_TU == 0
 #undef QM_PICK_0
 #define QM_PICK_0(...) QM_TILE_DEF(__VA_ARGS__)
@@ -222,6 +234,34 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16_11(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_11
 #define QM_PICK16S_11(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 12
+#undef QM_PICK_12
+#define QM_PICK_12(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_12
+#define QM_PICK16_12(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_12
+#define QM_PICK16S_12(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 13
+#undef QM_PICK_13
+#define QM_PICK_13(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_13
+#define QM_PICK16_13(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_13
+#define QM_PICK16S_13(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 14
+#undef QM_PICK_14
+#define QM_PICK_14(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_14
+#define QM_PICK16_14(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_14
+#define QM_PICK16S_14(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 15
+#undef QM_PICK_15
+#define QM_PICK_15(...) QM_TILE_DEF(__VA_ARGS__)
+#undef QM_PICK16_15
+#define QM_PICK16_15(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_15
+#define QM_PICK16S_15(...) QM_TILE16S_DEF(__VA_ARGS__)
 #else
 #error "QM_TU out of range"
 #endif
