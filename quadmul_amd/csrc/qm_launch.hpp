@@ -1,6 +1,7 @@
 // Host-side launch plumbing shared by the translation units of libqm_hip.so.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include "qm_common.hpp"
 
 namespace qm {
@@ -10,18 +11,20 @@ typedef hipError_t (*LaunchFn)(const GemmArgs &, hipStream_t, int group_m);
 
 constexpr int QM_MAX_DEVICES = 64;
 
-// Kernels that want more than 64 KiB of dynamic LDS must say so once per device.
+// Kernels that want more than 64 KiB of dynamic LDS must say so once per device.  (The
+// flags are atomics: several host threads may launch at once; setting the attribute twice
+// is harmless.)
 template <class KernelPtr>
-inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, bool *done_per_device)
+inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, std::atomic<bool> *done_per_device)
 {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= QM_MAX_DEVICES) return hipErrorInvalidDevice;
-    if (!done_per_device[dev]) {
+    if (!done_per_device[dev].load(std::memory_order_acquire)) {
         e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
         if (e != hipSuccess) return e;
-        done_per_device[dev] = true;
+        done_per_device[dev].store(true, std::memory_order_release);
     }
     return hipSuccess;
 }

@@ -15,7 +15,7 @@ namespace qm {
 template <class Cfg, class Kernel>
 static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
 {
-    static bool lds_ok[QM_MAX_DEVICES] = {};
+    static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
     hipError_t e = ensure_dynamic_lds(kernel, Cfg::LDS_BYTES, lds_ok);
     if (e != hipSuccess) return e;
     const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
@@ -34,15 +34,16 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 template <class Cfg, int OUT, class Kernel>
 static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
 {
-    static bool lds_ok[QM_MAX_DEVICES] = {};
-    static int resident[QM_MAX_DEVICES] = {};  // workgroups the device holds at once (0: not asked yet)
+    static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
+    static std::atomic<int> resident[QM_MAX_DEVICES] = {};  // workgroups the device holds at once (0: not asked yet)
     hipError_t e = ensure_dynamic_lds(kernel, Cfg::LDS_BYTES, lds_ok);
     if (e != hipSuccess) return e;
     int dev = 0;
     e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= QM_MAX_DEVICES) return hipErrorInvalidDevice;
-    if (resident[dev] == 0) {
+    int held = resident[dev].load(std::memory_order_acquire);
+    if (held == 0) {
         int per_cu = 0, cus = 0;
         e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, Cfg::THREADS, Cfg::LDS_BYTES);
         if (e != hipSuccess) return e;
@@ -51,7 +52,8 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
         if (per_cu < 1) per_cu = 1;
         // a multiple of 8, so that an item index modulo 8 names the XCD it runs on
         int g = per_cu * cus / 8 * 8;
-        resident[dev] = g < 8 ? 8 : g;
+        held = g < 8 ? 8 : g;
+        resident[dev].store(held, std::memory_order_release);
     }
     const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
     int group_m = opt & 0xFF, ksplit = (opt >> 8) & 0xFF;
@@ -66,7 +68,7 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
     const long long items = (long long)tiles_m * tiles_n * ksplit;
     if (items > 0x7FFFFFFF) return hipErrorInvalidValue;
     int grid = (int)items;
-    if (!(opt & 0x10000) && grid > resident[dev]) grid = resident[dev];
+    if (!(opt & 0x10000) && grid > held) grid = held;
     kernel<<<dim3(grid), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, tiles_m, tiles_n, group_m, ksplit);
     return hipGetLastError();
 }
