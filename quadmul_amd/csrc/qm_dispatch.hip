@@ -495,7 +495,7 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
     if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
     if (m <= 64) {
         const int fm = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
-        const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w8_u4p");
+        const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w16_u1");
         const int id = find_config(name);
         if (id >= 0) return {id, 1, 1};
     }

@@ -5,7 +5,8 @@
 // owns 16*FN rows of B (columns of C) and all of M (padded to 16*FM <= 128); its
 // NW waves split K between them in 128-nibble chunks, each wave streaming its
 // share of B straight from HBM into registers, and the partial 16x16 blocks are
-// summed through LDS.  One launch, no workspace, no atomics, C overwritten.
+// added up in the LDS with integer atomics.  One launch, no workspace, no global atomics,
+// C overwritten.
 //
 // The MFMA wants lane r + 16 g to hold 16 bytes of row r (k-group g), which as a
 // load has consecutive lanes in different rows: the memory pipeline then handles
@@ -27,7 +28,7 @@ struct SkinnyCfg {
     static constexpr int FM = FM_, FN = FN_, NW = NW_, U = U_, APF = APF_;
     static constexpr int THREADS = 64 * NW;
     static constexpr int MAX_M = 16 * FM, BN = 16 * FN;
-    static constexpr int LDS_BYTES = NW * FM * FN * 64 * 16;
+    static constexpr int LDS_BYTES = FM * FN * 64 * 16;  // one block set: the waves add into it
     static_assert(LDS_BYTES <= 64 * 1024, "static LDS");
 };
 
@@ -36,7 +37,9 @@ __global__ void __launch_bounds__(Cfg::THREADS)
 gemm_skinny_kernel(const GemmArgs p)
 {
     constexpr int FM = Cfg::FM, FN = Cfg::FN, NW = Cfg::NW, U = Cfg::U;
-    __shared__ v4i red[NW][FM * FN][64];
+    // the sum of the waves' partial blocks: [block][register e][lane], so that the 64 lanes
+    // of an LDS atomic fall into 64 consecutive words
+    __shared__ int32_t red[FM * FN][4][64];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, g = lane >> 4;
@@ -67,6 +70,9 @@ gemm_skinny_kernel(const GemmArgs p)
     for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+    // (cleared now, while the waves are still starting up; the barrier costs nothing yet)
+    for (int idx = tid; idx < FM * FN * 256; idx += Cfg::THREADS) (&red[0][0][0])[idx] = 0;
+    __syncthreads();
 
     // chunk c belongs to wave (c / U) % NW: each wave takes U consecutive chunks
     // per round so that its U*(FN+FM) loads are all in flight before the first MFMA.
@@ -127,23 +133,22 @@ gemm_skinny_kernel(const GemmArgs p)
         for (int u = 0; u < U; ++u) contract(bq[u], aq[u]);
     }
 
-    // ---- reduce the NW partial sums through LDS ----
+    // ---- add the NW partial sums up in the LDS (integer atomics: any order) ----
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) red[wave][i * FN + j][lane] = acc[i][j];
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                __hip_atomic_fetch_add(&red[i * FN + j][e][lane], acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     __syncthreads();
 
     // One output element per thread and pass: element (m, n) of block blk sits in register
-    // n % 4 of lane m + 16 * (n / 4) of every wave's partial block; 16 consecutive threads
-    // write 64 contiguous bytes of a row of C.
-    const int32_t *red_i = reinterpret_cast<const int32_t *>(&red[0][0][0]);
+    // n % 4 of lane m + 16 * (n / 4); 16 consecutive threads write 64 contiguous bytes of a
+    // row of C.
     for (int idx = tid; idx < FM * FN * 256; idx += Cfg::THREADS) {
         const int blk = idx >> 8, ml = (idx >> 4) & 15, nl = idx & 15;
-        const int src = (blk * 64 + ml + 16 * (nl >> 2)) * 4 + (nl & 3);
-        int32_t s = 0;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) s += red_i[w * (FM * FN * 256) + src];
+        const int32_t s = red[blk][nl & 3][ml + 16 * (nl >> 2)];
         const int m = (blk / FN) * 16 + ml, n = n0 + (blk % FN) * 16 + nl;
         if (m < p.M && n < p.N) {
             const size_t at = (size_t)m * p.N + n;
