@@ -387,6 +387,15 @@ static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
     hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U>>(p, s, gm); }
 #define QM_SKINNYP(FM, FN, NW, U) \
     hipError_t QM_SKINNYP_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U, 1>>(p, s, gm); }
+template <class Cfg>
+static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int)
+{
+    const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
+    gemm_dot_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), 0, stream>>>(p);
+    return hipGetLastError();
+}
+#define QM_DOT(MR, FN, NW, U) \
+    hipError_t QM_DOT_FN(MR, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_dot<DotCfg<MR, FN, NW, U>>(p, s, gm); }
 #include "qm_configs.inc"
 
 // --------------------------------------------------------------------------
@@ -419,6 +428,9 @@ static const ConfigDesc g_configs[] = {
 #define QM_SKINNYP(FM, FN, NW, U)                                                     \
     {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U) "p", KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
      &QM_SKINNYP_FN(FM, FN, NW, U)},
+#define QM_DOT(MR, FN, NW, U)                                                     \
+    {"v" QM_STR(MR) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, MR, 16 * (FN), 128, NW, 0, \
+     &QM_DOT_FN(MR, FN, NW, U)},
 #include "qm_configs.inc"
 };
 static constexpr int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
@@ -493,6 +505,10 @@ struct Choice {
 static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
 {
     if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
+    if (m <= 2) {
+        const int id = find_config(m == 1 ? "v1x1_w8_u4" : "v2x1_w16_u2");
+        if (id >= 0) return {id, 1, 1};
+    }
     if (m <= 64) {
         const int fm = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
         const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w16_u1");

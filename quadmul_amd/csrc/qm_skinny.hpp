@@ -158,4 +158,94 @@ gemm_skinny_kernel(const GemmArgs p)
     }
 }
 
+// --------------------------------------------------------------------------
+// One or two rows of A (GEMV-like shapes): no matrix core.  v_dot8_i32_i4 multiplies eight
+// signed nibbles of one dword with the eight of another and adds them up -- the packed
+// format as it is, no widening, no lane permutation, no factor to shift away.  A workgroup
+// owns 16 * FN rows of B and all of M; its NW waves split K in 128-nibble chunks as above;
+// a lane loads 16 bytes of row lane / 4 of B (coalesced quads) and the matching 16 bytes
+// of every row of A (the same 64 bytes for all 16 quads of the wave: one cache line),
+// and the four lanes of a quad add their sums up at the end.  Measured against the matrix-core
+// kernel at N = K = 4096: 2.3 us against 3.0 us for one row, 2.5 against 3.0 for two, even
+// from three rows on (the dot instructions then take as long as the lane permutations).
+// --------------------------------------------------------------------------
+template <int MR_, int FN_, int NW_, int U_>
+struct DotCfg {
+    static constexpr int MR = MR_, FN = FN_, NW = NW_, U = U_;
+    static constexpr int THREADS = 64 * NW;
+    static constexpr int MAX_M = MR, BN = 16 * FN;
+};
+
+template <class Cfg>
+__global__ void __launch_bounds__(Cfg::THREADS)
+gemm_dot_kernel(const GemmArgs p)
+{
+    constexpr int MR = Cfg::MR, FN = Cfg::FN, NW = Cfg::NW, U = Cfg::U;
+    __shared__ int32_t red[MR][FN * 16];  // the sum over the waves
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n0 = blockIdx.x * Cfg::BN;
+    const int Kb = p.K >> 1;
+    const int nchunks = (p.K + 127) >> 7;
+    const int ld_row = lane >> 2, ld_ch = lane & 3;
+    uint32_t b_off[FN], a_off[MR];
+#pragma unroll
+    for (int j = 0; j < FN; ++j) b_off[j] = (uint32_t)min(n0 + j * 16 + ld_row, p.N - 1) * (uint32_t)Kb + ld_ch * 16;
+#pragma unroll
+    for (int i = 0; i < MR; ++i) a_off[i] = (uint32_t)min(i, p.M - 1) * (uint32_t)Kb + ld_ch * 16;
+
+    int32_t acc[MR][FN];
+#pragma unroll
+    for (int i = 0; i < MR; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = 0;
+    for (int idx = tid; idx < MR * FN * 16; idx += Cfg::THREADS) (&red[0][0])[idx] = 0;
+    __syncthreads();
+
+    for (int c0 = wave * U; c0 < nchunks; c0 += NW * U) {
+        v4i bq[U][FN], aq[U][MR];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int kofs = (c0 + u) * 64;
+            const bool ok = kofs + ld_ch * 16 < Kb;  // also false for c0+u >= nchunks; zeros add nothing
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                bq[u][j] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p.B + b_off[j] + kofs)) : v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < MR; ++i)
+                aq[u][i] = ok ? *reinterpret_cast<const v4i *>(p.A + a_off[i] + kofs) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < MR; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][j] = __builtin_amdgcn_sdot8(aq[u][i][e], bq[u][j][e], acc[i][j], false);
+    }
+
+    // the four lanes of a quad hold the four 32-nibble pieces of a chunk: add them up, then
+    // the waves' sums in the LDS
+#pragma unroll
+    for (int i = 0; i < MR; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            int32_t v = acc[i][j];
+            v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+            v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+            if (ld_ch == 0) __hip_atomic_fetch_add(&red[i][j * 16 + ld_row], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    __syncthreads();
+    for (int idx = tid; idx < MR * FN * 16; idx += Cfg::THREADS) {
+        const int m = idx / (FN * 16), n = n0 + idx % (FN * 16);
+        if (m < p.M && n < p.N) {
+            const int32_t s = (&red[0][0])[idx];
+            const size_t at = (size_t)m * p.N + n;
+            if (p.out == OUT_I32) p.C[at] = s;
+            else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
+        }
+    }
+}
+
 }  // namespace qm

@@ -122,7 +122,7 @@ def test_config_registry():
     names = qm.config_names()
     assert names[0] == "generic" and len(names) == len(set(names))
     assert any(n.startswith("t256x256") for n in names) and any(n.startswith("s1x1") for n in names)
-    assert any(n.startswith("q256x256") for n in names)
+    assert any(n.startswith("q256x256") for n in names) and any(n.startswith("v1x1") for n in names)
     for i, n in enumerate(names):
         assert qm.config_id(n) == i
     with pytest.raises(qm.QuadmulError):
@@ -134,8 +134,9 @@ def test_selection_rules():
     assert name(8192, 8192, 8192).startswith("q")   # pipelined 16x16x64 kernel: K % 128 == 0
     assert name(4096, 4096, 4096).startswith("q")
     assert name(4096, 4096, 4096 + 32).startswith("t")  # K % 32 == 0 only: plain tile kernel
-    for m in (1, 16, 64):
+    for m in (16, 64):
         assert name(m, 4096, 4096).startswith("s"), m
+    assert name(1, 4096, 4096).startswith("v") and name(2, 5120, 5120).startswith("v")   # dot-product kernel
     # few tiles, long K: the pipelined kernel with K split over several workgroups per tile
     code = qm.select_config(128, 8192, 28672)
     assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1

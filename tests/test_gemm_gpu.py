@@ -428,3 +428,27 @@ def test_random_shapes_through_the_automatic_choice():
         seen.add(name[0] + ("+split" if (code >> 24) & 0x3F > 1 else ""))
         assert torch.equal(c_d, want), f"{m}x{n}x{k} ({name}, ksplit {(code >> 24) & 0x3F})"
     assert {"g", "s", "t", "q", "q+split"} <= seen, seen
+
+
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (2, 4100, 11008), (1, 50, 131040), (2, 33, 28672), (1, 4096, 96)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_dot_product_kernel_one_and_two_rows(oracle_mod, shape):
+    """The GEMV-like kernel (v_dot8_i32_i4 on the packed nibbles as they are): random data
+    against the oracle, the extremes in closed form, on every such configuration."""
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 5500 + n)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    lo_a = pack_cpu(torch.full((m, k), -8, dtype=torch.int8))
+    lo_b, hi_b = pack_cpu(torch.full((n, k), -8, dtype=torch.int8)), pack_cpu(torch.full((n, k), 7, dtype=torch.int8))
+    ran = 0
+    for cfg, name in enumerate(qm.config_names()):
+        if not name.startswith("v") or not qm.config_supports(cfg, m, n, k):
+            continue
+        assert oracle_mod.compare(run_gemm(ap, bp, m, n, k, cfg), want) == -1, name
+        assert (run_gemm(lo_a, lo_b, m, n, k, cfg) == 64 * k).all(), name
+        assert (run_gemm(lo_a, hi_b, m, n, k, cfg) == -56 * k).all(), name
+        ran += 1
+    assert ran >= (2 if m == 1 else 1)
+    assert qm.config_name(qm.select_config(m, n, k) & 0xFFFF).startswith("v")
+    assert oracle_mod.compare(run_gemm(ap, bp, m, n, k), want) == -1
