@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the packed-int4 GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload square4096|square8192|skinny16]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload square4096|square8192|skinny16|skinny1]
 
 A step is one call of ``quadmul.gemm`` (the drop-in entry point) on operands already
 resident in HBM.  Prints ONE JSON line: the throughput of the main workload
@@ -34,6 +34,7 @@ WORKLOADS = {
     "square4096": (1, 4096, 4096, 4096, "mfma"),
     "square8192": (8, 8192, 8192, 8192, "mfma"),
     "skinny16": (3, 16, 4096, 4096, "hbm"),
+    "skinny1": (2, 1, 4096, 4096, "hbm"),
 }
 
 
