@@ -279,6 +279,20 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         }
     };
 
+    // The same in two halves, two MFMA slots apart, for the K loop: the LDS address goes into
+    // M0 first (the slots in between are the wait state the load needs after a write of M0),
+    // the load itself follows alone -- five instructions in one slot are more than the shadow
+    // of that slot's MFMA hides.  Nothing else in this kernel uses M0.
+    auto dma_setup = [&](int piece, int stage_byte) __attribute__((always_inline)) {
+        const uint32_t dst = dma_lds + stage_byte +
+                             (piece < A_PIECES ? piece * WAVES * 16 * PITCH : Cfg::A_BYTES + (piece - A_PIECES) * WAVES * 16 * PITCH);
+        asm volatile("s_mov_b32 m0, %0" ::"s"(dst) : "memory", "m0");
+    };
+    auto dma_issue = [&](int piece) __attribute__((always_inline)) {
+        if (piece < A_PIECES) asm volatile("global_load_lds_dwordx4 %0, %1" ::"v"(a_goff[piece]), "s"(a_src) : "memory");
+        else asm volatile("global_load_lds_dwordx4 %0, %1" ::"v"(b_goff[piece - A_PIECES]), "s"(b_src) : "memory");
+    };
+
     // ---- fragment reads: lane -> row r of a 16-row fragment, chunk g (32 nibbles) ----
     // (rows of consecutive fragments differ by 16, which leaves (row >> 1) & 3 unchanged)
     const int a_row = wm * Cfg::WM + r, b_row = wn * Cfg::WN + r;
@@ -535,13 +549,25 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 // -- write-out of the accumulator row finished one sub-step ago --
                 if constexpr (last && i >= 1) write_whole(std::integral_constant<int, i - 1>{}, s_);
                 // -- DMA pieces of the step AHEAD of this one, one sub-step apart --
+                // (With a ring of three stages the loads issued in a step must have landed
+                // at its end.  In a last step they all go out in sub-step 0, ahead of the
+                // first store, so that "all but the stores" can be waited for.)
+                constexpr bool bunched = last && AHEAD == 2;
+                constexpr bool split = !bunched && NP <= FM && SLOTS >= 4;  // at most one piece per sub-step
+                if constexpr (split && s == SLOTS - 3) {
+                    static_for<0, NP>([&](auto q_) {
+                        constexpr int q = decltype(q_)::value;
+                        if constexpr (q * FM / NP == i) dma_setup(q, ring[STAGES - 1]);
+                    });
+                }
                 if constexpr (s == SLOTS - 1) {
                     static_for<0, NP>([&](auto q_) {
                         constexpr int q = decltype(q_)::value;
-                        // (With a ring of three stages the loads issued in a step must have landed
-                        // at its end.  In a last step they all go out in sub-step 0, ahead of the
-                        // first store, so that "all but the stores" can be waited for.)
-                        if constexpr (last && AHEAD == 2 ? i == 0 : q * FM / NP == i) dma_piece(q, ring[STAGES - 1]);
+                        if constexpr (split) {
+                            if constexpr (q * FM / NP == i) dma_issue(q);
+                        } else if constexpr (bunched ? i == 0 : q * FM / NP == i) {
+                            dma_piece(q, ring[STAGES - 1]);
+                        }
                     });
                 }
                 __builtin_amdgcn_sched_barrier(0);
