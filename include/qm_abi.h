@@ -95,7 +95,11 @@ int qm_config_has_scaled(int cfg); /* 1 / 0 */
  * faster with K split over several workgroups per tile; with a workspace each split
  * stores its partial tile there with plain 16-byte stores and a second kernel adds the
  * splits up (scaling and rounding, for the scaled form), instead of 4-byte atomics into
- * C.  Results are identical to the forms without a workspace.
+ * C.  The second use (cfg = QM_CFG_AUTO only): large shapes whose K is not a multiple of
+ * 128, or whose operands are not 16-byte aligned, get copies of A and B in the workspace
+ * with every row padded with zeros to whole 128-nibble steps, and run on the pipelined
+ * kernel instead of the plain tile / generic kernels (about a quarter faster at
+ * 8192 x 8192 x 8224).  Results are identical to the forms without a workspace.
  *   workspace        device memory, 16-byte aligned, or NULL; used by the kernels of this
  *                    call only (in stream order): calls that may overlap on the GPU need
  *                    a workspace each, calls on one stream can share one
@@ -106,7 +110,7 @@ int qm_config_has_scaled(int cfg); /* 1 / 0 */
  * cfg as for qm_gemm_i4_cfg (QM_CFG_AUTO included); with a workspace the scaled form also
  * takes K splits, on every "q" configuration.
  * qm_gemm_workspace_bytes: what the call with these arguments uses at most (0 when it
- * would not split K); scaled = 1 for the scaled form.
+ * needs none); scaled = 1 for the scaled form.
  */
 int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg,
                   void *workspace, size_t workspace_bytes);

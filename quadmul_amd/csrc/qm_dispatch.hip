@@ -79,6 +79,32 @@ __global__ void fill_zero_kernel(int32_t *dst, size_t n)
 }
 
 // --------------------------------------------------------------------------
+// Operand copy with every row padded with zeros to a whole number of 128-nibble K-steps
+// (zero nibbles add nothing to a product): what lets the pipelined kernel run shapes whose
+// K is not a multiple of 128, or whose operands are not 16-byte aligned, out of a
+// caller-provided workspace.  kb / kbp: bytes per row of the source / of the copy.
+// --------------------------------------------------------------------------
+__global__ void pad_rows_vec_kernel(const v4i *__restrict__ src, v4i *__restrict__ dst, int rows, int kb16, int kbp16)
+{
+    const size_t total = (size_t)rows * kbp16;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / kbp16;
+        const int c = (int)(i - r * kbp16);
+        dst[i] = c < kb16 ? src[r * kb16 + c] : v4i{0, 0, 0, 0};
+    }
+}
+
+__global__ void pad_rows_byte_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int rows, int kb, int kbp)
+{
+    const size_t total = (size_t)rows * kbp;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / kbp;
+        const int c = (int)(i - r * kbp);
+        dst[i] = c < kb ? src[r * kb + c] : (uint8_t)0;
+    }
+}
+
+// --------------------------------------------------------------------------
 // K split with a workspace (pipelined kernel): item (split s, tile t) of the GEMM launch
 // left its BM x BN partial sums in slot s * ntiles + t, wave by wave, block by block, 16
 // bytes per lane in the order the MFMA leaves a block (lane l: row l % 16, columns
@@ -544,7 +570,7 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         const int kt = (k + 127) / 128;
         auto cost_of = [&](int ks_) {
             double rounds = (double)((tiles * ks_ + 255) / 256);
-            if (d.kind == KIND_TILE) rounds = std::max((double)tiles / 256.0, c.share);
+            if (d.kind == KIND_TILE && c.share > 1.0) rounds = std::max((double)tiles / 256.0, c.share);
             return rounds * (double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + (d.kind == KIND_TILE ? 120000.0 : std::ceil(rounds) * 240000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
         };
         int ks = 1;
@@ -659,6 +685,68 @@ static bool workspace_fits(const ConfigDesc &d, int m, int n, int ksplit, const 
     return ws != nullptr && ((uintptr_t)ws & 15) == 0 && ws_bytes >= split_workspace_bytes(d, m, n, ksplit);
 }
 
+// Automatic choice only: K padded to a multiple of 128 (operands copied into the workspace) so
+// that the pipelined kernel can run.  Worth it when the shape is large -- the copy is
+// (M + N) K / 2 bytes twice over, the plain tile kernels are about a third slower than the
+// pipelined one, the generic kernel many times.  `direct` is the choice without padding.
+struct PadPlan {
+    bool on = false;
+    int kp = 0;
+    Choice ch{};
+    size_t a_bytes = 0, b_bytes = 0;
+    size_t bytes() const { return a_bytes + b_bytes; }
+};
+
+static PadPlan plan_padded_k(int m, int n, int k, int ptr_align, const Choice &direct)
+{
+    PadPlan pl;
+    const int kind = g_configs[direct.cfg].kind;
+    if (kind == KIND_TILE16 || kind == KIND_SKINNY) return pl;
+    const int kp = (k + 127) / 128 * 128;
+    if (kp > QM_MAX_K_X16 || !fast_path_ok(m, n, kp, 256)) return pl;
+    const long long outs = (long long)m * n;
+    if (kind == KIND_TILE ? outs < 4096LL * 2048 : outs * k < (1LL << 27)) return pl;
+    (void)ptr_align;
+    Choice ch = heuristic(m, n, kp, 256, false);
+    // (instead of a plain tile kernel only the pipelined one pays; instead of the generic
+    // kernel anything does)
+    if (kind == KIND_TILE ? g_configs[ch.cfg].kind != KIND_TILE16 : g_configs[ch.cfg].kind == KIND_GENERIC) return pl;
+    ch.ksplit = 1;
+    pl.on = true;
+    pl.kp = kp;
+    pl.ch = ch;
+    pl.a_bytes = ((size_t)m * (kp / 2) + 255) / 256 * 256;
+    pl.b_bytes = ((size_t)n * (kp / 2) + 255) / 256 * 256;
+    return pl;
+}
+
+static hipError_t launch_pad_rows(const void *src, void *dst, int rows, int k, int kp, hipStream_t s)
+{
+    const int kb = k / 2, kbp = kp / 2;
+    if (kb % 16 == 0 && ((uintptr_t)src & 15) == 0) {
+        const size_t total = (size_t)rows * (kbp / 16);
+        pad_rows_vec_kernel<<<dim3(flat_grid(total, 256)), dim3(256), 0, s>>>(static_cast<const v4i *>(src), static_cast<v4i *>(dst), rows, kb / 16, kbp / 16);
+    } else {
+        const size_t total = (size_t)rows * kbp;
+        pad_rows_byte_kernel<<<dim3(flat_grid(total, 256)), dim3(256), 0, s>>>(static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), rows, kb, kbp);
+    }
+    return hipGetLastError();
+}
+
+// The padded copies of A and B in the workspace, and the arguments of the GEMM on them.
+static hipError_t launch_padded(GemmArgs &p, const PadPlan &pl, void *ws, hipStream_t s)
+{
+    uint8_t *a_p = static_cast<uint8_t *>(ws), *b_p = a_p + pl.a_bytes;
+    hipError_t e = launch_pad_rows(p.A, a_p, p.M, p.K, pl.kp, s);
+    if (e != hipSuccess) return e;
+    e = launch_pad_rows(p.B, b_p, p.N, p.K, pl.kp, s);
+    if (e != hipSuccess) return e;
+    p.A = a_p;
+    p.B = b_p;
+    p.K = pl.kp;
+    return hipSuccess;
+}
+
 static Choice choice_from_code(int cfg)
 {
     Choice ch;
@@ -733,7 +821,15 @@ QM_EXPORT int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n,
         if (ch.ksplit > 1 && g_configs[ch.cfg].kind != KIND_TILE16) return QM_ERR_CONFIG;
     }
     ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
-    const GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(C), m, n, k};
+    GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(C), m, n, k};
+    if (cfg == QM_CFG_AUTO && has_ws) {
+        const PadPlan pl = plan_padded_k(m, n, k, align, ch);
+        if (pl.on && ((uintptr_t)workspace & 15) == 0 && workspace_bytes >= pl.bytes()) {
+            hipError_t e = launch_padded(p, pl, workspace, s);
+            if (e == hipSuccess) e = g_configs[pl.ch.cfg].launch(p, s, pl.ch.group_m | (1 << 8) | (pl.ch.spread << 16));
+            return e == hipSuccess ? QM_OK : fail_launch(e);
+        }
+    }
     if (ch.ksplit > 1 && workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) {
         const hipError_t e = launch_split_with_workspace(p, ch, workspace, s);
         return e == hipSuccess ? QM_OK : fail_launch(e);
@@ -797,6 +893,19 @@ QM_EXPORT int qm_gemm_i4_scaled_ws(const void *A, const void *B, void *D, int m,
         const hipError_t e = launch_split_with_workspace(p, ch, workspace, s);
         return e == hipSuccess ? QM_OK : fail_launch(e);
     }
+    if (cfg == QM_CFG_AUTO && has_ws) {
+        PadPlan pl = plan_padded_k(m, n, k, align, ch);
+        if (pl.on && !scaled_launcher(pl.ch.cfg)) {
+            // a pipelined configuration that has the scaled output, if the shape is one for those
+            const int id = find_config(g_configs[pl.ch.cfg].kind == KIND_TILE16 ? "q256x256_w2x2_s4o1" : "q128x128_w2x2_s4o1");
+            if (id >= 0) pl.ch.cfg = id; else pl.on = false;
+        }
+        if (pl.on && ((uintptr_t)workspace & 15) == 0 && workspace_bytes >= pl.bytes()) {
+            hipError_t e = launch_padded(p, pl, workspace, s);
+            if (e == hipSuccess) e = scaled_launcher(pl.ch.cfg)(p, s, pl.ch.group_m | (1 << 8) | (pl.ch.spread << 16));
+            return e == hipSuccess ? QM_OK : fail_launch(e);
+        }
+    }
     const LaunchFn launch = scaled_launcher(ch.cfg);
     if (!launch) return QM_ERR_CONFIG;
     const hipError_t e = launch(p, s, ch.group_m | (1 << 8) | (ch.spread << 16));
@@ -826,7 +935,12 @@ QM_EXPORT size_t qm_gemm_workspace_bytes(int m, int n, int k, int ptr_align, int
         if (!config_supports(ch.cfg, m, n, k, ptr_align)) return 0;
     }
     const int ks = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
-    return ks > 1 ? split_workspace_bytes(g_configs[ch.cfg], m, n, ks) : 0;
+    if (ks > 1) return split_workspace_bytes(g_configs[ch.cfg], m, n, ks);
+    if (cfg == QM_CFG_AUTO) {
+        const PadPlan pl = plan_padded_k(m, n, k, ptr_align, ch);
+        if (pl.on) return pl.bytes();
+    }
+    return 0;
 }
 
 QM_EXPORT int qm_config_has_scaled(int cfg)

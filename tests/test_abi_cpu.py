@@ -116,6 +116,10 @@ def test_workspace_sizes():
     assert qm.workspace_bytes(128, 8192, 28672) == qm.workspace_bytes(128, 8192, 28672, code) > 0
     assert qm.workspace_bytes(128, 8192, 28672, scaled=True) > 0
     assert qm.workspace_bytes(0, 8192, 28672) == 0 and qm.workspace_bytes(128, 8192, 3) == 0
+    # large shapes with K % 128 != 0: room for copies of A and B with rows padded to whole K-steps
+    assert qm.workspace_bytes(4096, 4096, 4160) == 2 * 4096 * (4224 // 2)
+    assert qm.workspace_bytes(512, 4096, 2752) == 0          # too small to pay for the copies
+    assert qm.workspace_bytes(4096, 4096, 4160, qm.config_id("t256x256x128_w4x2_m0")) == 0   # explicit configuration: as asked
 
 
 def test_config_registry():

@@ -452,3 +452,38 @@ def test_dot_product_kernel_one_and_two_rows(oracle_mod, shape):
     assert ran >= (2 if m == 1 else 1)
     assert qm.config_name(qm.select_config(m, n, k) & 0xFFFF).startswith("v")
     assert oracle_mod.compare(run_gemm(ap, bp, m, n, k), want) == -1
+
+
+@pytest.mark.parametrize("shape", [(3000, 3000, 1056), (1000, 1000, 1000), (300, 5000, 4098), (2100, 4200, 96 + 2)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_k_padded_through_the_workspace(shape):
+    """Large shapes whose K is not a multiple of 128 (or 32), and unaligned operands: with a
+    workspace the operands are copied with zero-padded rows and the pipelined kernel runs;
+    without one the plain tile / generic kernels do.  Same result, against an exact fp32 matmul."""
+    import quadmul
+
+    m, n, k = shape
+    a = torch.randint(-8, 8, (m, k), dtype=torch.int8, generator=torch.Generator().manual_seed(SEED_BASE + 5600 + k))
+    b = torch.randint(-8, 8, (n, k), dtype=torch.int8, generator=torch.Generator().manual_seed(SEED_BASE + 5700 + k))
+    want = fp32_matmul_on_gpu(a, b)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    assert qm.workspace_bytes(m, n, k) >= (m + n) * ((k + 127) // 128 * 64)
+    for fn in (lambda c: quadmul.gemm(a_d, b_d, c, m, n, k), lambda c: qm.gemm(a_d, b_d, c, m, n, k),
+               lambda c: qm.gemm(a_d, b_d, c, m, n, k, workspace=None),
+               lambda c: qm.gemm(a_d, b_d, c, m, n, k, workspace=torch.empty(4096, dtype=torch.uint8, device=DEV))):
+        c_d = poisoned_c(m, n, DEV)
+        fn(c_d)
+        torch.cuda.synchronize()
+        assert torch.equal(c_d, want)
+    # operands at odd addresses
+    a_buf = torch.empty(ap.numel() + 1, dtype=torch.int8, device=DEV)
+    b_buf = torch.empty(bp.numel() + 3, dtype=torch.int8, device=DEV)
+    a_odd, b_odd = a_buf[1:].view(m, k // 2), b_buf[3:].view(n, k // 2)
+    a_odd.copy_(a_d)
+    b_odd.copy_(b_d)
+    assert a_odd.data_ptr() % 2 == 1
+    c_d = poisoned_c(m, n, DEV)
+    qm.gemm(a_odd, b_odd, c_d, m, n, k)
+    torch.cuda.synchronize()
+    assert torch.equal(c_d, want)

@@ -229,3 +229,20 @@ def test_scaled_random_shapes_through_the_automatic_choice():
         qm.gemm_scaled(a_d, b_d, d, m, n, k, rs_d, cs_d)
         torch.cuda.synchronize()
         assert torch.equal(d.view(torch.int16), want.view(torch.int16)), f"{m}x{n}x{k} {dtype}"
+
+
+def test_scaled_k_padded_through_the_workspace():
+    m, n, k = 3000, 3000, 1056
+    a = torch.randint(-8, 8, (m, k), dtype=torch.int8, generator=torch.Generator().manual_seed(SEED_BASE + 7600))
+    b = torch.randint(-8, 8, (n, k), dtype=torch.int8, generator=torch.Generator().manual_seed(SEED_BASE + 7700))
+    rs, cs = make_scales(m, n, SEED_BASE + 7800)
+    a_d, b_d, rs_d, cs_d = pack_cpu(a).to(DEV), pack_cpu(b).to(DEV), rs.to(DEV), cs.to(DEV)
+    c32 = a.to(DEV).float() @ b.to(DEV).float().t()
+    assert qm.workspace_bytes(m, n, k, scaled=True) > 0
+    for dtype in (torch.float16, torch.bfloat16):
+        want = ((c32 * rs_d[:, None]) * cs_d[None, :]).to(dtype)
+        for ws in (True, None):
+            d = poisoned_d(m, n, dtype)
+            qm.gemm_scaled(a_d, b_d, d, m, n, k, rs_d, cs_d, workspace=ws)
+            torch.cuda.synchronize()
+            assert torch.equal(d.view(torch.int16), want.view(torch.int16)), (dtype, ws)
