@@ -549,7 +549,8 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
     // this is priced as if it had this many.
     static const struct { const char *name; double eff, share; } cands[] = {
         {"q256x256_w2x2_s4o1", 1.00, 1.0}, {"q256x128_w2x2_s4o1", 0.82, 1.0}, {"q128x256_w2x2_s4o1", 0.82, 1.0},
-        {"q128x128_w2x2_s4o1", 0.60, 1.0}, {"t256x256x128_w4x2_m0", 0.70, 1.0}, {"t128x128x128_w2x2_m0", 0.35, 1.0},
+        {"q128x128_w2x2_s4o1", 0.60, 1.0}, {"q128x64_w2x2_s4o2", 0.46, 1.0}, {"q64x128_w2x2_s4o2", 0.44, 1.0},
+        {"q64x64_w2x2_s4o2", 0.37, 1.0}, {"t256x256x128_w4x2_m0", 0.70, 1.0}, {"t128x128x128_w2x2_m0", 0.35, 1.0},
         {"t64x128x128_w2x2_m0", 0.27, 1.5}, {"t128x64x128_w2x2_m0", 0.27, 1.5}, {"t64x64x128_w2x2_m0", 0.28, 2.0},
     };
     int best = 0, best_ks = 1;

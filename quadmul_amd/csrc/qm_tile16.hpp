@@ -143,6 +143,7 @@ struct Tile16Cfg {
     static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
     static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
     static_assert((W_OPS * FN) % FM == 0, "B widening must split evenly over the sub-steps");
+    static_assert(FN <= 2 * FM, "at most two B fragments are read per sub-step (two packed registers)");
 };
 
 template <class Cfg, int OUT = OUT_I32>
