@@ -629,8 +629,9 @@ static Choice select_scaled(int m, int n, int k, int ptr_align, bool has_ws)
             if (id < 0) continue;
             const ConfigDesc &d = g_configs[id];
             const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
-            const double eff = d.bm * d.bn >= 256 * 256 ? 1.0 : (d.bm * d.bn >= 256 * 128 ? 0.82 : 0.66);
-            const double cost = (double)((tiles + 255) / 256) * d.bm * d.bn / eff;
+            const int area = d.bm * d.bn;
+            const double eff = area >= 256 * 256 ? 1.0 : (area >= 256 * 128 ? 0.82 : (area >= 128 * 128 ? 0.60 : (area >= 128 * 64 ? 0.45 : 0.37)));
+            const double cost = (double)((tiles + 255) / 256) * ((double)((k + 127) / 128) * area / eff + 240000.0);  // as in heuristic()
             if (cost < best_cost) { best_cost = cost; best = id; }
         }
         if (best >= 0) return {best, 4, 1};
