@@ -96,10 +96,10 @@ int qm_config_has_scaled(int cfg); /* 1 / 0 */
  * stores its partial tile there with plain 16-byte stores and a second kernel adds the
  * splits up (scaling and rounding, for the scaled form), instead of 4-byte atomics into
  * C.  The second use (cfg = QM_CFG_AUTO only): large shapes whose K is not a multiple of
- * 128, or whose operands are not 16-byte aligned, get copies of A and B in the workspace
+ * 32, or whose operands are not 16-byte aligned, get copies of A and B in the workspace
  * with every row padded with zeros to whole 128-nibble steps, and run on the pipelined
- * kernel instead of the plain tile / generic kernels (about a quarter faster at
- * 8192 x 8192 x 8224).  Results are identical to the forms without a workspace.
+ * kernel instead of the generic one.  Results are identical to the forms without a
+ * workspace.
  *   workspace        device memory, 16-byte aligned, or NULL; used by the kernels of this
  *                    call only (in stream order): calls that may overlap on the GPU need
  *                    a workspace each, calls on one stream can share one

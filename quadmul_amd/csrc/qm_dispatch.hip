@@ -504,7 +504,7 @@ static bool config_supports(int cfg, int m, int n, int k, int ptr_align)
     if (c.kind == KIND_GENERIC) return true;
     if (!fast_path_ok(m, n, k, ptr_align)) return false;
     if (c.kind == KIND_SKINNY) return m <= c.bm;
-    if (c.kind == KIND_TILE16) return k % 128 == 0;  // whole K-steps only: its loop has no tail path
+    if (c.kind == KIND_TILE16) return k % 128 == 0 || k > 128;  // a short last K-step needs a step before it
     return true;
 }
 
@@ -672,8 +672,7 @@ static int fail_launch(hipError_t e)
 static int effective_ksplit(const ConfigDesc &d, int k, int ksplit)
 {
     if (d.kind != KIND_TILE16 || ksplit <= 1) return 1;
-    const int kt = k / d.bk, kps = (kt + ksplit - 1) / ksplit;
-    return (kt + kps - 1) / kps;
+    return normalised_ksplit(k, ksplit);
 }
 
 static size_t split_workspace_bytes(const ConfigDesc &d, int m, int n, int ksplit)

@@ -11,6 +11,22 @@ typedef hipError_t (*LaunchFn)(const GemmArgs &, hipStream_t, int group_m);
 
 constexpr int QM_MAX_DEVICES = 64;
 
+// K split of the pipelined kernel, normalised: kt K-steps of 128 nibbles (the last one may
+// be short); with kps steps per split only ceil(kt / kps) splits have work; and a split
+// that holds a short last step keeps at least two steps (the kernel widens that step's B
+// operand during the step before it, inside the same work item).
+inline int normalised_ksplit(int K, int ksplit)
+{
+    const int kt = (K + 127) / 128;
+    if (ksplit < 1) ksplit = 1;
+    for (;;) {
+        const int kps = (kt + ksplit - 1) / ksplit;
+        ksplit = (kt + kps - 1) / kps;
+        if (ksplit == 1 || (K & 127) == 0 || kt - (ksplit - 1) * kps >= 2) return ksplit;
+        --ksplit;
+    }
+}
+
 // Kernels that want more than 64 KiB of dynamic LDS must say so once per device.  (The
 // flags are atomics: several host threads may launch at once; setting the attribute twice
 // is harmless.)

@@ -144,9 +144,12 @@ struct Tile16Cfg {
     static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
     static_assert((W_OPS * FN) % FM == 0, "B widening must split evenly over the sub-steps");
     static_assert(FN <= 2 * FM, "at most two B fragments are read per sub-step (two packed registers)");
+    static_assert(FN <= 2 * FM, "at most two B fragments are read per sub-step (two packed registers)");
 };
 
-template <class Cfg, int OUT = OUT_I32>
+// TAIL: K % 128 may be 32, 64 or 96 (a short last K-step); the instantiation without it is
+// the same kernel with that code left out.
+template <class Cfg, int OUT = OUT_I32, bool TAIL = false>
 __global__ void __launch_bounds__(Cfg::THREADS, Cfg::OCC * Cfg::THREADS / 256)
 gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const int group_m, const int ksplit)
 {
@@ -176,7 +179,12 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     const int ntiles = tiles_m * tiles_n;
     const int nitems = ntiles * ksplit;
     const int Kb = p.K >> 1;
-    const int kt_all = p.K / BK;  // K is a multiple of 128 for this kernel
+    // K is a multiple of 128, or with TAIL of 32.  A last K-step of fewer than 128 nibbles
+    // (K % 128 = 32, 64 or 96) is loaded as the last 128 nibbles of the row -- in bounds,
+    // 16-byte aligned -- and the part of it that the step before already covered is masked
+    // away in the widening of B.
+    const int kt_all = TAIL ? (p.K + BK - 1) / BK : p.K / BK;
+    const int k_tail = TAIL ? (p.K & (BK - 1)) >> 5 : 0;  // valid 32-nibble chunks of that step, 0: none short
     const int kps = (kt_all + ksplit - 1) / ksplit;
 
     // item -> tile origin and K-step range [kt0, kt0 + KT); KT >= 1 (the launcher never
@@ -246,7 +254,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     };
     const uint8_t *a_src, *b_src;  // operand base + K offset of the step the cursor points at
     auto cursor_point = [&]() __attribute__((always_inline)) {
-        const int kofs = (d_kt0 + min(d_kt, d_KT - 1)) * (BK / 2);
+        const int step = d_kt0 + min(d_kt, d_KT - 1);
+        const int kofs = (TAIL && k_tail != 0 && step == kt_all - 1) ? Kb - BK / 2 : step * (BK / 2);
         a_src = p.A + kofs;
         b_src = p.B + kofs;
     };
@@ -361,6 +370,14 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // an SGPR operand is half the size of one with a 32-bit literal.
     uint32_t amask;
     asm volatile("s_mov_b32 %0, 0xf0f0f0f0" : "=s"(amask));
+    // TAIL: B's mask is a vector register: all nibbles, none (an item's padding step), or per
+    // lane for a short last step -- lane (r, g) holds chunk g of the step, and of the 128
+    // nibbles loaded for that step the first 4 - k_tail chunks belong to the step before.
+    uint32_t vmask_full = 0, vmask_tail = 0;
+    if constexpr (TAIL) {
+        asm volatile("v_mov_b32 %0, 0xf0f0f0f0" : "=v"(vmask_full));
+        vmask_tail = (k_tail == 0 || g >= 4 - k_tail) ? vmask_full : 0u;
+    }
 
     // ---- writing a finished tile ----
     // A 16x16 block leaves the MFMA with lane (r, g) holding row r, columns 4g..4g+3: a
@@ -621,14 +638,31 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
 #pragma unroll
                 for (int e = 0; e < 4; ++e) keep_here_f(cs_reg[j][e]);
         }
-        for (c_kt = 0; c_kt + 2 < c_KT; c_kt += 2) {
-            k_step(amask, std::integral_constant<int, 0>{}, std::false_type{});
-            k_step(amask, std::integral_constant<int, 1>{}, std::false_type{});
-        }
-        // (the mask is made opaque: knowing it is either all-ones-per-nibble or zero, the
+        // (the masks are made opaque: knowing one to be all-ones-per-nibble or zero, the
         // compiler would hoist the whole widening of B out of the MFMA slots into a branch)
-        uint32_t bmask = c_kt + 1 < c_KT ? amask : 0u;
-        asm volatile("" : "+s"(bmask));
+        uint32_t bmask, full;
+        if constexpr (TAIL) {
+            // the step of this item that is the short last step of K, or -1 (the launcher sees to
+            // it that such an item has at least two steps: its B is widened inside the item)
+            const int tail_at = (k_tail != 0 && c_kt0 + c_KT == kt_all) ? c_KT - 1 : -1;
+            for (c_kt = 0; c_kt + 2 < c_KT; c_kt += 2) {
+                k_step(vmask_full, std::integral_constant<int, 0>{}, std::false_type{});
+                uint32_t m2 = c_kt + 2 == tail_at ? vmask_tail : vmask_full;
+                asm volatile("" : "+v"(m2));
+                k_step(m2, std::integral_constant<int, 1>{}, std::false_type{});
+            }
+            bmask = c_kt + 1 < c_KT ? (c_kt + 1 == tail_at ? vmask_tail : vmask_full) : 0u;
+            asm volatile("" : "+v"(bmask));
+            full = vmask_full;
+        } else {
+            for (c_kt = 0; c_kt + 2 < c_KT; c_kt += 2) {
+                k_step(amask, std::integral_constant<int, 0>{}, std::false_type{});
+                k_step(amask, std::integral_constant<int, 1>{}, std::false_type{});
+            }
+            bmask = c_kt + 1 < c_KT ? amask : 0u;
+            asm volatile("" : "+s"(bmask));
+            full = amask;
+        }
         tile_c = reinterpret_cast<char *>(p.C) + ((size_t)c_m0 * p.N + c_n0) * ESZ;
         if constexpr (OUT == OUT_I32 && !whole) {
             // workspace slot of a K-split item: (split, tile) in the order locate() numbers them
@@ -637,7 +671,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                            ((size_t)xcd_contiguous_id(c_item, nitems) * WAVES + wave) * (FM * FN * 64) + lane;
         }
         k_step(bmask, std::integral_constant<int, 0>{}, std::false_type{});
-        k_step(amask, std::integral_constant<int, 1>{}, std::integral_constant<bool, whole>{});
+        k_step(full, std::integral_constant<int, 1>{}, std::integral_constant<bool, whole>{});
         // Let the last MFMAs retire before their accumulators are read (the compiler does not
         // know the asm statements were MFMAs, so the wait is tied to the accumulators written
         // last and cannot be scheduled around); then the rows not written out yet.

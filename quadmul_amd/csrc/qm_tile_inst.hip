@@ -31,7 +31,8 @@ static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t str
 // default the grid is persistent: as many workgroups as the device holds at once, each
 // running several (K split, tile) items back to back.
 // (OUT is a template parameter so that every kernel gets launcher statics of its own.)
-template <class Cfg, int OUT, class Kernel>
+// (... and TAIL: the kernel for K % 128 != 0 is another kernel with statics of its own)
+template <class Cfg, int OUT, bool TAIL, class Kernel>
 static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
 {
     static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
@@ -59,12 +60,7 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
     int group_m = opt & 0xFF, ksplit = (opt >> 8) & 0xFF;
     if (group_m < 1) group_m = 1;
     if (group_m > tiles_m) group_m = tiles_m;
-    if (ksplit < 1) ksplit = 1;
-    {
-        // no empty splits: with kps K-steps per split, only ceil(kt / kps) splits have work
-        const int kt = p.K / Cfg::BK, kps = (kt + ksplit - 1) / ksplit;
-        ksplit = (kt + kps - 1) / kps;
-    }
+    ksplit = normalised_ksplit(p.K, ksplit);
     const long long items = (long long)tiles_m * tiles_n * ksplit;
     if (items > 0x7FFFFFFF) return hipErrorInvalidValue;
     int grid = (int)items;
@@ -88,7 +84,8 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
     hipError_t QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &p, hipStream_t s, int gm) \
     {                                                                                            \
         using Cfg = Tile16Cfg<BM, BN, WGM, WGN, ST, OCC>;                                        \
-        return launch_tiled_persistent<Cfg, OUT_I32>(&gemm_tile16_kernel<Cfg, OUT_I32>, p, s, gm);  \
+        if (p.K % 128) return launch_tiled_persistent<Cfg, OUT_I32, true>(&gemm_tile16_kernel<Cfg, OUT_I32, true>, p, s, gm); \
+        return launch_tiled_persistent<Cfg, OUT_I32, false>(&gemm_tile16_kernel<Cfg, OUT_I32, false>, p, s, gm);  \
     }                                                                                            \
     }
 // the same configuration with the scaled 16-bit float outputs
@@ -97,8 +94,12 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
     hipError_t QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &p, hipStream_t s, int gm) \
     {                                                                                             \
         using Cfg = Tile16Cfg<BM, BN, WGM, WGN, ST, OCC>;                                         \
-        if (p.out == OUT_F16) return launch_tiled_persistent<Cfg, OUT_F16>(&gemm_tile16_kernel<Cfg, OUT_F16>, p, s, gm); \
-        return launch_tiled_persistent<Cfg, OUT_BF16>(&gemm_tile16_kernel<Cfg, OUT_BF16>, p, s, gm); \
+        if (p.K % 128) {                                                                            \
+            if (p.out == OUT_F16) return launch_tiled_persistent<Cfg, OUT_F16, true>(&gemm_tile16_kernel<Cfg, OUT_F16, true>, p, s, gm); \
+            return launch_tiled_persistent<Cfg, OUT_BF16, true>(&gemm_tile16_kernel<Cfg, OUT_BF16, true>, p, s, gm); \
+        }                                                                                           \
+        if (p.out == OUT_F16) return launch_tiled_persistent<Cfg, OUT_F16, false>(&gemm_tile16_kernel<Cfg, OUT_F16, false>, p, s, gm); \
+        return launch_tiled_persistent<Cfg, OUT_BF16, false>(&gemm_tile16_kernel<Cfg, OUT_BF16, false>, p, s, gm); \
     }                                                                                             \
     }
 

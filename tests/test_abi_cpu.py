@@ -70,7 +70,7 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4(None, None, None, 4, 0, 4, None) == 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 4, 4, 4, None, 9999) == -3
     assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("t128x128x128_w2x2_m0")) == -3
-    assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 160, None, qm.config_id("q256x256_w2x2_s4o1")) == -3
+    assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 96, None, qm.config_id("q256x256_w2x2_s4o1")) == -3   # a single short K-step
     assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
     assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
     assert lib.qm_unpack_i4(None, one, 4, 8, None) == -1
@@ -116,10 +116,13 @@ def test_workspace_sizes():
     assert qm.workspace_bytes(128, 8192, 28672) == qm.workspace_bytes(128, 8192, 28672, code) > 0
     assert qm.workspace_bytes(128, 8192, 28672, scaled=True) > 0
     assert qm.workspace_bytes(0, 8192, 28672) == 0 and qm.workspace_bytes(128, 8192, 3) == 0
-    # large shapes with K % 128 != 0: room for copies of A and B with rows padded to whole K-steps
-    assert qm.workspace_bytes(4096, 4096, 4160) == 2 * 4096 * (4224 // 2)
-    assert qm.workspace_bytes(512, 4096, 2752) == 0          # too small to pay for the copies
-    assert qm.workspace_bytes(4096, 4096, 4160, qm.config_id("t256x256x128_w4x2_m0")) == 0   # explicit configuration: as asked
+    # large shapes with K % 32 != 0 (or unaligned operands): room for copies of A and B with rows
+    # padded to whole K-steps
+    assert qm.workspace_bytes(4096, 4096, 4162) == 2 * 4096 * (4224 // 2)
+    assert qm.workspace_bytes(4096, 4096, 4160, ptr_align=2) == 2 * 4096 * (4224 // 2)
+    assert qm.workspace_bytes(4096, 4096, 4160) == 0         # K % 32 == 0: the pipelined kernel takes it as it is
+    assert qm.workspace_bytes(60, 70, 4162) == 0             # too small to pay for the copies
+    assert qm.workspace_bytes(4096, 4096, 4162, qm.config_id("generic")) == 0   # explicit configuration: as asked
 
 
 def test_config_registry():
@@ -137,7 +140,8 @@ def test_selection_rules():
     name = lambda m, n, k, al=256: qm.config_name(qm.select_config(m, n, k, al) & 0xFFFF)
     assert name(8192, 8192, 8192).startswith("q")   # pipelined 16x16x64 kernel: K % 128 == 0
     assert name(4096, 4096, 4096).startswith("q")
-    assert name(4096, 4096, 4096 + 32).startswith("t")  # K % 32 == 0 only: plain tile kernel
+    assert name(4096, 4096, 4096 + 32).startswith("q")  # K % 32 == 0: the pipelined kernel with a short last K-step
+    assert name(4096, 4096, 96).startswith("t")         # a single short K-step: plain tile kernel
     for m in (16, 64):
         assert name(m, 4096, 4096).startswith("s"), m
     assert name(1, 4096, 4096).startswith("v") and name(2, 5120, 5120).startswith("v")   # dot-product kernel

@@ -457,9 +457,10 @@ def test_dot_product_kernel_one_and_two_rows(oracle_mod, shape):
 @pytest.mark.parametrize("shape", [(3000, 3000, 1056), (1000, 1000, 1000), (300, 5000, 4098), (2100, 4200, 96 + 2)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_k_padded_through_the_workspace(shape):
-    """Large shapes whose K is not a multiple of 128 (or 32), and unaligned operands: with a
-    workspace the operands are copied with zero-padded rows and the pipelined kernel runs;
-    without one the plain tile / generic kernels do.  Same result, against an exact fp32 matmul."""
+    """Large shapes whose K is not a multiple of 32, and unaligned operands: with a workspace
+    the operands are copied with zero-padded rows and the pipelined kernel runs; without one
+    the generic kernel does.  (K % 32 == 0, first case: no copies, a short last K-step.)  Same
+    result, against an exact fp32 matmul."""
     import quadmul
 
     m, n, k = shape
@@ -468,7 +469,10 @@ def test_k_padded_through_the_workspace(shape):
     want = fp32_matmul_on_gpu(a, b)
     ap, bp = pack_cpu(a), pack_cpu(b)
     a_d, b_d = ap.to(DEV), bp.to(DEV)
-    assert qm.workspace_bytes(m, n, k) >= (m + n) * ((k + 127) // 128 * 64)
+    if k % 32:
+        assert qm.workspace_bytes(m, n, k) >= (m + n) * ((k + 127) // 128 * 64)
+    else:   # K % 32 == 0: the pipelined kernel runs it as it is, with a short last K-step
+        assert qm.workspace_bytes(m, n, k) == 0 and qm.config_name(qm.select_config(m, n, k) & 0xFFFF).startswith("q")
     for fn in (lambda c: quadmul.gemm(a_d, b_d, c, m, n, k), lambda c: qm.gemm(a_d, b_d, c, m, n, k),
                lambda c: qm.gemm(a_d, b_d, c, m, n, k, workspace=None),
                lambda c: qm.gemm(a_d, b_d, c, m, n, k, workspace=torch.empty(4096, dtype=torch.uint8, device=DEV))):
@@ -487,3 +491,29 @@ def test_k_padded_through_the_workspace(shape):
     qm.gemm(a_odd, b_odd, c_d, m, n, k)
     torch.cuda.synchronize()
     assert torch.equal(c_d, want)
+
+
+@pytest.mark.parametrize("k", [160, 192, 224, 288, 4128, 4160, 4192, 11040], ids=lambda k: f"k{k}")
+def test_short_last_k_step_on_every_pipelined_config(oracle_mod, k):
+    """K % 128 = 32, 64, 96: the last K-step of the pipelined kernel is loaded as the last 128
+    nibbles of the row and the overlap with the step before is masked; whole and ragged tiles,
+    K splits (the split that holds the short step keeps two steps), both item orders."""
+    m, n = 300, 520
+    a, b = make_operands(m, n, k, SEED_BASE + 5800 + k)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    hi_a, lo_b = pack_cpu(torch.full((m, k), 7, dtype=torch.int8)), pack_cpu(torch.full((n, k), -8, dtype=torch.int8))
+    ran = 0
+    for cfg, name in enumerate(qm.config_names()):
+        if not name.startswith("q"):
+            continue
+        assert qm.config_supports(cfg, m, n, k), name
+        for gm, ks, spread in [(1, 1, 0), (4, 1, 1), (2, 2, 0), (3, 3, 0), (1, 16, 0)]:
+            code = cfg | (gm << 16) | (ks << 24) | (spread << 30)
+            for ws in ([True, None] if ks > 1 else [True]):
+                got = run_gemm(ap, bp, m, n, k, code, ws)
+                bad = oracle_mod.compare(got, want)
+                assert bad == -1, f"{name} group_m={gm} ksplit={ks} spread={spread} workspace={ws}: first mismatch at flat index {bad}"
+        assert (run_gemm(hi_a, lo_b, m, n, k, cfg) == -56 * k).all(), name   # every nibble counted exactly once
+        ran += 1
+    assert ran >= 8

@@ -232,7 +232,7 @@ def test_scaled_random_shapes_through_the_automatic_choice():
 
 
 def test_scaled_k_padded_through_the_workspace():
-    m, n, k = 3000, 3000, 1056
+    m, n, k = 3000, 3000, 1058
     a = torch.randint(-8, 8, (m, k), dtype=torch.int8, generator=torch.Generator().manual_seed(SEED_BASE + 7600))
     b = torch.randint(-8, 8, (n, k), dtype=torch.int8, generator=torch.Generator().manual_seed(SEED_BASE + 7700))
     rs, cs = make_scales(m, n, SEED_BASE + 7800)
