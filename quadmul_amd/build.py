@@ -28,7 +28,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 OBJDIR = os.path.join(PKG, "build")
 LIB_PATH = os.path.join(LIBDIR, "libqm_hip.so")
-N_TILE_TUS = 14
+N_TILE_TUS = 12
 
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [

@@ -427,7 +427,7 @@ static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int)
 // --------------------------------------------------------------------------
 // Configuration registry
 // --------------------------------------------------------------------------
-enum Kind { KIND_GENERIC = 0, KIND_TILE = 1, KIND_SKINNY = 2, KIND_TILE16 = 3 };
+enum Kind { KIND_GENERIC = 0, KIND_SKINNY = 2, KIND_TILE16 = 3 };
 
 struct ConfigDesc {
     const char *name;
@@ -442,9 +442,6 @@ struct ConfigDesc {
 #define QM_STR(x) QM_STR2(x)
 static const ConfigDesc g_configs[] = {
     {"generic", KIND_GENERIC, 16, 16, 128, 4, 0, &launch_generic},
-#define QM_TILE(tu, BM, BN, BK, WGM, WGN, MODE)                                                        \
-    {"t" QM_STR(BM) "x" QM_STR(BN) "x" QM_STR(BK) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_m" QM_STR(MODE), \
-     KIND_TILE, BM, BN, BK, (WGM) * (WGN), MODE, &QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)},
 #define QM_TILE16(tu, BM, BN, WGM, WGN, ST, OCC)                                                              \
     {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_s" QM_STR(ST) "o" QM_STR(OCC), KIND_TILE16, BM, BN, 128, \
      (WGM) * (WGN), 0, &QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC), WGM, WGN},
@@ -469,8 +466,8 @@ static const struct { const char *name; LaunchFn launch; } g_scaled_tile16[] = {
 };
 
 // The launcher of configuration cfg for the scaled output, or null: the generic and the
-// skinny kernels take the output form at run time, the pipelined ones as separate kernels,
-// the plain tile kernels not at all.
+// skinny kernels take the output form at run time, the pipelined ones as separate kernels
+// (not every configuration has them).
 static LaunchFn scaled_launcher(int cfg)
 {
     const ConfigDesc &c = g_configs[cfg];
@@ -543,15 +540,10 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
     }
     // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency),
     // over the configurations that can run this K.  Efficiencies are measured ratios.
-    // eff: throughput per tile area relative to the 256 x 256 pipelined kernel with the GPU
-    // full.  share: the plain tile kernels run several small workgroups per CU, and one
-    // alone does not run that many times faster -- a launch with fewer tiles per CU than
-    // this is priced as if it had this many.
-    static const struct { const char *name; double eff, share; } cands[] = {
-        {"q256x256_w2x2_s4o1", 1.00, 1.0}, {"q256x128_w2x2_s4o1", 0.82, 1.0}, {"q128x256_w2x2_s4o1", 0.82, 1.0},
-        {"q128x128_w2x2_s4o1", 0.60, 1.0}, {"q128x64_w2x2_s4o2", 0.46, 1.0}, {"q64x128_w2x2_s4o2", 0.44, 1.0},
-        {"q64x64_w2x2_s4o2", 0.37, 1.0}, {"t256x256x128_w4x2_m0", 0.70, 1.0}, {"t128x128x128_w2x2_m0", 0.35, 1.0},
-        {"t64x128x128_w2x2_m0", 0.27, 1.5}, {"t128x64x128_w2x2_m0", 0.27, 1.5}, {"t64x64x128_w2x2_m0", 0.28, 2.0},
+    // eff: throughput per tile area relative to the 256 x 256 tile with the GPU full (measured)
+    static const struct { const char *name; double eff; } cands[] = {
+        {"q256x256_w2x2_s4o1", 1.00}, {"q256x128_w2x2_s4o1", 0.82}, {"q128x256_w2x2_s4o1", 0.82}, {"q128x128_w2x2_s4o1", 0.60},
+        {"q128x64_w2x2_s4o2", 0.46},  {"q64x128_w2x2_s4o2", 0.44},  {"q64x64_w2x2_s4o2", 0.37},
     };
     int best = 0, best_ks = 1;
     double best_cost = 1e300;
@@ -566,13 +558,12 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         // enough that splitting only pays when each split keeps a long K of its own
         // (measured: wins at K = 28672, loses at K = 8192).
         // Cost in units of 16.5 ps (one K-step of the 256 x 256 tile = 65536): K-steps per
-        // item x tile area / efficiency, plus 4 us per round of workgroups (2 us for the plain tile kernels) for filling the
+        // item x tile area / efficiency, plus 4 us per round of workgroups for filling the
         // ring and writing out, plus the split's own cost.
         const int kt = (k + 127) / 128;
         auto cost_of = [&](int ks_) {
-            double rounds = (double)((tiles * ks_ + 255) / 256);
-            if (d.kind == KIND_TILE && c.share > 1.0) rounds = std::max((double)tiles / 256.0, c.share);
-            return rounds * (double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + (d.kind == KIND_TILE ? 120000.0 : std::ceil(rounds) * 240000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
+            const double rounds = (double)((tiles * ks_ + 255) / 256);
+            return rounds * ((double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + 240000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
         };
         int ks = 1;
         double cost = cost_of(1);
@@ -687,9 +678,8 @@ static bool workspace_fits(const ConfigDesc &d, int m, int n, int ksplit, const 
 }
 
 // Automatic choice only: K padded to a multiple of 128 (operands copied into the workspace) so
-// that the pipelined kernel can run.  Worth it when the shape is large -- the copy is
-// (M + N) K / 2 bytes twice over, the plain tile kernels are about a third slower than the
-// pipelined one, the generic kernel many times.  `direct` is the choice without padding.
+// that the pipelined kernel can run instead of the generic one.  Worth it when the shape is
+// large -- the copy is (M + N) K / 2 bytes twice over.  `direct` is the choice without padding.
 struct PadPlan {
     bool on = false;
     int kp = 0;
@@ -706,12 +696,10 @@ static PadPlan plan_padded_k(int m, int n, int k, int ptr_align, const Choice &d
     const int kp = (k + 127) / 128 * 128;
     if (kp > QM_MAX_K_X16 || !fast_path_ok(m, n, kp, 256)) return pl;
     const long long outs = (long long)m * n;
-    if (kind == KIND_TILE ? outs < 4096LL * 2048 : outs * k < (1LL << 27)) return pl;
+    if (outs * k < (1LL << 27)) return pl;
     (void)ptr_align;
     Choice ch = heuristic(m, n, kp, 256, false);
-    // (instead of a plain tile kernel only the pipelined one pays; instead of the generic
-    // kernel anything does)
-    if (kind == KIND_TILE ? g_configs[ch.cfg].kind != KIND_TILE16 : g_configs[ch.cfg].kind == KIND_GENERIC) return pl;
+    if (g_configs[ch.cfg].kind == KIND_GENERIC) return pl;
     ch.ksplit = 1;
     pl.on = true;
     pl.kp = kp;

@@ -1,7 +1,6 @@
 // Instantiates the tile kernels assigned to translation unit QM_TU (see
 // qm_configs.inc); compiled once per unit so the build runs in parallel.
 #include "qm_launch.hpp"
-#include "qm_tile.hpp"
 #include "qm_tile16.hpp"
 
 #ifndef QM_TU
@@ -10,24 +9,9 @@
 
 namespace qm {
 
-// opt: tile raster group height in bits 0..7, K split in bits 8..15 (pipelined kernel only;
-// the caller has zero-filled C when the split is above 1)
-template <class Cfg, class Kernel>
-static hipError_t launch_tiled(Kernel kernel, const GemmArgs &p, hipStream_t stream, int opt)
-{
-    static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
-    hipError_t e = ensure_dynamic_lds(kernel, Cfg::LDS_BYTES, lds_ok);
-    if (e != hipSuccess) return e;
-    const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
-    int group_m = opt & 0xFF;
-    if (group_m < 1) group_m = 1;
-    if (group_m > tiles_m) group_m = tiles_m;
-    kernel<<<dim3(tiles_m * tiles_n), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, tiles_m, tiles_n, group_m);
-    return hipGetLastError();
-}
-
-// Pipelined kernel: opt additionally holds the K split in bits 8..15 (the caller has
-// zero-filled C when it is above 1) and, in bit 16, "one work item per workgroup".  By
+// opt: tile raster group height in bits 0..7, the K split in bits 8..15 (the caller has
+// zero-filled C, or given the kernel a workspace, when it is above 1) and, in bit 16, "one
+// work item per workgroup".  By
 // default the grid is persistent: as many workgroups as the device holds at once, each
 // running several (K split, tile) items back to back.
 // (OUT is a template parameter so that every kernel gets launcher statics of its own.)
@@ -71,14 +55,6 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 
 }  // namespace qm
 
-#define QM_TILE_DEF(BM, BN, BK, WGM, WGN, MODE)                                                 \
-    namespace qm {                                                                              \
-    hipError_t QM_TILE_FN(BM, BN, BK, WGM, WGN, MODE)(const GemmArgs &p, hipStream_t s, int gm) \
-    {                                                                                           \
-        using Cfg = TileCfg<BM, BN, BK, WGM, WGN, MODE>;                                        \
-        return launch_tiled<Cfg>(&gemm_tile_kernel<Cfg>, p, s, gm);                             \
-    }                                                                                           \
-    }
 #define QM_TILE16_DEF(BM, BN, WGM, WGN, ST, OCC)                                                 \
     namespace qm {                                                                               \
     hipError_t QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &p, hipStream_t s, int gm) \
@@ -105,22 +81,6 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 
 // An entry of qm_configs.inc is compiled here only when its unit number equals QM_TU:
 // QM_PICK*_<n> expands to nothing except for n == QM_TU.
-#define QM_PICK_0(...)
-#define QM_PICK_1(...)
-#define QM_PICK_2(...)
-#define QM_PICK_3(...)
-#define QM_PICK_4(...)
-#define QM_PICK_5(...)
-#define QM_PICK_6(...)
-#define QM_PICK_7(...)
-#define QM_PICK_8(...)
-#define QM_PICK_9(...)
-#define QM_PICK_10(...)
-#define QM_PICK_11(...)
-#define QM_PICK_12(...)
-#define QM_PICK_13(...)
-#define QM_PICK_14(...)
-#define QM_PICK_15(...)
 #define QM_PICK16_0(...)
 #define QM_PICK16_1(...)
 #define QM_PICK16_2(...)
@@ -133,10 +93,6 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16_9(...)
 #define QM_PICK16_10(...)
 #define QM_PICK16_11(...)
-#define QM_PICK16_12(...)
-#define QM_PICK16_13(...)
-#define QM_PICK16_14(...)
-#define QM_PICK16_15(...)
 #define QM_PICK16S_0(...)
 #define QM_PICK16S_1(...)
 #define QM_PICK16S_2(...)
@@ -149,127 +105,70 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16S_9(...)
 #define QM_PICK16S_10(...)
 #define QM_PICK16S_11(...)
-#define QM_PICK16S_12(...)
-#define QM_PICK16S_13(...)
-#define QM_PICK16S_14(...)
-#define QM_PICK16S_15(...)
 #if QM_TU == 0
-#undef QM_PICK_0
-#define QM_PICK_0(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_0
 #define QM_PICK16_0(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_0
 #define QM_PICK16S_0(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 1
-#undef QM_PICK_1
-#define QM_PICK_1(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_1
 #define QM_PICK16_1(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_1
 #define QM_PICK16S_1(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 2
-#undef QM_PICK_2
-#define QM_PICK_2(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_2
 #define QM_PICK16_2(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_2
 #define QM_PICK16S_2(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 3
-#undef QM_PICK_3
-#define QM_PICK_3(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_3
 #define QM_PICK16_3(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_3
 #define QM_PICK16S_3(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 4
-#undef QM_PICK_4
-#define QM_PICK_4(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_4
 #define QM_PICK16_4(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_4
 #define QM_PICK16S_4(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 5
-#undef QM_PICK_5
-#define QM_PICK_5(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_5
 #define QM_PICK16_5(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_5
 #define QM_PICK16S_5(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 6
-#undef QM_PICK_6
-#define QM_PICK_6(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_6
 #define QM_PICK16_6(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_6
 #define QM_PICK16S_6(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 7
-#undef QM_PICK_7
-#define QM_PICK_7(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_7
 #define QM_PICK16_7(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_7
 #define QM_PICK16S_7(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 8
-#undef QM_PICK_8
-#define QM_PICK_8(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_8
 #define QM_PICK16_8(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_8
 #define QM_PICK16S_8(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 9
-#undef QM_PICK_9
-#define QM_PICK_9(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_9
 #define QM_PICK16_9(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_9
 #define QM_PICK16S_9(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 10
-#undef QM_PICK_10
-#define QM_PICK_10(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_10
 #define QM_PICK16_10(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_10
 #define QM_PICK16S_10(...) QM_TILE16S_DEF(__VA_ARGS__)
 #elif QM_TU == 11
-#undef QM_PICK_11
-#define QM_PICK_11(...) QM_TILE_DEF(__VA_ARGS__)
 #undef QM_PICK16_11
 #define QM_PICK16_11(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_11
 #define QM_PICK16S_11(...) QM_TILE16S_DEF(__VA_ARGS__)
-#elif QM_TU == 12
-#undef QM_PICK_12
-#define QM_PICK_12(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_12
-#define QM_PICK16_12(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK16S_12
-#define QM_PICK16S_12(...) QM_TILE16S_DEF(__VA_ARGS__)
-#elif QM_TU == 13
-#undef QM_PICK_13
-#define QM_PICK_13(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_13
-#define QM_PICK16_13(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK16S_13
-#define QM_PICK16S_13(...) QM_TILE16S_DEF(__VA_ARGS__)
-#elif QM_TU == 14
-#undef QM_PICK_14
-#define QM_PICK_14(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_14
-#define QM_PICK16_14(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK16S_14
-#define QM_PICK16S_14(...) QM_TILE16S_DEF(__VA_ARGS__)
-#elif QM_TU == 15
-#undef QM_PICK_15
-#define QM_PICK_15(...) QM_TILE_DEF(__VA_ARGS__)
-#undef QM_PICK16_15
-#define QM_PICK16_15(...) QM_TILE16_DEF(__VA_ARGS__)
-#undef QM_PICK16S_15
-#define QM_PICK16S_15(...) QM_TILE16S_DEF(__VA_ARGS__)
 #else
 #error "QM_TU out of range"
 #endif
 
-#define QM_TILE(tu, ...) QM_PICK_##tu(__VA_ARGS__)
 #define QM_TILE16(tu, ...) QM_PICK16_##tu(__VA_ARGS__)
 #define QM_TILE16S(tu, ...) QM_PICK16S_##tu(__VA_ARGS__)
 #include "qm_configs.inc"

@@ -69,7 +69,7 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4(None, None, None, 0, 4, 4, None) == 0    # empty: nothing to do
     assert lib.qm_gemm_i4(None, None, None, 4, 0, 4, None) == 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 4, 4, 4, None, 9999) == -3
-    assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("t128x128x128_w2x2_m0")) == -3
+    assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("q128x128_w2x2_s4o1")) == -3   # K % 32 != 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 96, None, qm.config_id("q256x256_w2x2_s4o1")) == -3   # a single short K-step
     assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
     assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
@@ -80,7 +80,7 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4_scaled(one, one, None, 4, 4, 4, None, None, 1, None) == -1
     assert lib.qm_gemm_i4_scaled(one, one, ctypes.c_void_p(4097), 4, 4, 4, None, None, 2, None) == -5
     assert lib.qm_gemm_i4_scaled(None, None, None, 0, 4, 4, None, None, 1, None) == 0
-    assert lib.qm_gemm_i4_scaled_cfg(one, one, one, 64, 64, 128, None, None, 1, None, qm.config_id("t64x64x128_w2x2_m0")) == -3
+    assert lib.qm_gemm_i4_scaled_cfg(one, one, one, 64, 64, 128, None, None, 1, None, qm.config_id("q256x256_w2x4_s4o1")) == -3   # no scaled output
     assert lib.qm_gemm_i4_scaled_cfg(one, one, one, 256, 256, 256, None, None, 1, None, qm.config_id("q256x256_w2x2_s4o1") | (2 << 24)) == -3
     assert lib.qm_quantize_pack_i4(one, 9, one, one, 4, 8, None) == -6
     assert lib.qm_quantize_pack_i4(one, 1, one, one, 4, 7, None) == -2
@@ -91,12 +91,12 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4_ws(one, one, one, 4, 4, 3, None, -1, None, 0) == -2
     assert lib.qm_gemm_i4_ws(one, one, None, 4, 4, 4, None, -1, one, 1 << 20) == -1
     assert lib.qm_gemm_i4_ws(None, None, None, 0, 4, 4, None, -1, None, 0) == 0
-    assert lib.qm_gemm_i4_ws(one, one, one, 64, 64, 512, None, qm.config_id("t64x64x128_w2x2_m0") | (2 << 24), one, 1 << 20) == -3
+    assert lib.qm_gemm_i4_ws(one, one, one, 64, 64, 512, None, qm.config_id("s4x1_w8_u2") | (2 << 24), one, 1 << 20) == -3   # only the pipelined kernel splits K
     assert lib.qm_gemm_i4_scaled_ws(one, one, one, 4, 4, 4, None, None, 7, None, -1, None, 0) == -6
     assert lib.qm_gemm_i4_scaled_ws(one, one, one, 256, 256, 512, None, None, 1, None, qm.config_id("q256x256_w2x2_s4o1") | (2 << 24), one, 4096) == -3
     has = [qm.config_has_scaled(i) for i in range(qm.num_configs())]
     assert has[qm.config_id("generic")] and has[qm.config_id("q256x256_w2x2_s4o1")] and has[qm.config_id("s1x1_w8_u4")]
-    assert not has[qm.config_id("t64x64x128_w2x2_m0")] and not has[qm.config_id("q256x128_w2x2_s3o2")]
+    assert not has[qm.config_id("q256x256_w2x4_s4o1")] and not has[qm.config_id("q256x128_w2x2_s3o2")]
     for code in (0, -1, -2, -3, -4, -5, -6):
         assert lib.qm_status_string(code)
     assert b"gfx950" in lib.qm_version()
@@ -109,7 +109,7 @@ def test_workspace_sizes():
     # splits without work do not count: 3 K-steps cannot feed 8 splits
     assert qm.workspace_bytes(200, 300, 384, q128 | (8 << 24)) == 3 * 6 * 128 * 128 * 4
     assert qm.workspace_bytes(200, 300, 4096, q128) == 0                       # no split asked for
-    assert qm.workspace_bytes(200, 300, 4096, qm.config_id("t128x128x128_w2x2_m0") | (4 << 24)) == 0
+    assert qm.workspace_bytes(16, 300, 4096, qm.config_id("s1x1_w8_u4") | (4 << 24)) == 0
     assert qm.workspace_bytes(8192, 8192, 8192) == 0                           # plenty of tiles
     code = qm.select_config(128, 8192, 28672)
     assert (code >> 24) & 0x3F > 1
@@ -128,7 +128,7 @@ def test_workspace_sizes():
 def test_config_registry():
     names = qm.config_names()
     assert names[0] == "generic" and len(names) == len(set(names))
-    assert any(n.startswith("t256x256") for n in names) and any(n.startswith("s1x1") for n in names)
+    assert any(n.startswith("q64x64") for n in names) and any(n.startswith("s1x1") for n in names)
     assert any(n.startswith("q256x256") for n in names) and any(n.startswith("v1x1") for n in names)
     for i, n in enumerate(names):
         assert qm.config_id(n) == i
@@ -141,7 +141,7 @@ def test_selection_rules():
     assert name(8192, 8192, 8192).startswith("q")   # pipelined 16x16x64 kernel: K % 128 == 0
     assert name(4096, 4096, 4096).startswith("q")
     assert name(4096, 4096, 4096 + 32).startswith("q")  # K % 32 == 0: the pipelined kernel with a short last K-step
-    assert name(4096, 4096, 96).startswith("t")         # a single short K-step: plain tile kernel
+    assert name(4096, 4096, 96) == "generic"            # a single short K-step: nothing for the pipelined kernel to overlap it with
     for m in (16, 64):
         assert name(m, 4096, 4096).startswith("s"), m
     assert name(1, 4096, 4096).startswith("v") and name(2, 5120, 5120).startswith("v")   # dot-product kernel
