@@ -411,8 +411,6 @@ static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
 }
 #define QM_SKINNY(FM, FN, NW, U) \
     hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U>>(p, s, gm); }
-#define QM_SKINNYP(FM, FN, NW, U) \
-    hipError_t QM_SKINNYP_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U, 1>>(p, s, gm); }
 template <class Cfg>
 static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int)
 {
@@ -448,9 +446,6 @@ static const ConfigDesc g_configs[] = {
 #define QM_SKINNY(FM, FN, NW, U)                                                     \
     {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
      &QM_SKINNY_FN(FM, FN, NW, U)},
-#define QM_SKINNYP(FM, FN, NW, U)                                                     \
-    {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U) "p", KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
-     &QM_SKINNYP_FN(FM, FN, NW, U)},
 #define QM_DOT(MR, FN, NW, U)                                                     \
     {"v" QM_STR(MR) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, MR, 16 * (FN), 128, NW, 0, \
      &QM_DOT_FN(MR, FN, NW, U)},

@@ -46,7 +46,6 @@ inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, std::atomic<bo
 }
 
 #define QM_SKINNY_FN(FM, FN, NW, U) qm_launch_skinny_##FM##_##FN##_##NW##_##U
-#define QM_SKINNYP_FN(FM, FN, NW, U) qm_launch_skinnyp_##FM##_##FN##_##NW##_##U
 #define QM_DOT_FN(MR, FN, NW, U) qm_launch_dot_##MR##_##FN##_##NW##_##U
 #define QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC) qm_launch_tile16_##BM##_##BN##_##WGM##_##WGN##_##ST##_##OCC
 #define QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC) qm_launch_tile16s_##BM##_##BN##_##WGM##_##WGN##_##ST##_##OCC
@@ -54,7 +53,6 @@ inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, std::atomic<bo
 #define QM_TILE16(tu, BM, BN, WGM, WGN, ST, OCC) hipError_t QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &, hipStream_t, int);
 #define QM_TILE16S(tu, BM, BN, WGM, WGN, ST, OCC) hipError_t QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &, hipStream_t, int);
 #define QM_SKINNY(FM, FN, NW, U) hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &, hipStream_t, int);
-#define QM_SKINNYP(FM, FN, NW, U) hipError_t QM_SKINNYP_FN(FM, FN, NW, U)(const GemmArgs &, hipStream_t, int);
 #define QM_DOT(MR, FN, NW, U) hipError_t QM_DOT_FN(MR, FN, NW, U)(const GemmArgs &, hipStream_t, int);
 #include "qm_configs.inc"
 

@@ -19,13 +19,9 @@
 
 namespace qm {
 
-// APF = 0: the A and B loads of U chunks are all in flight before the first MFMA (few rows
-// of A: the loads are few).  APF = 1, for M up to 128: the B loads of U chunks are in flight
-// at once -- they come from HBM -- while A, which the L2 holds, is loaded one chunk ahead of
-// the MFMAs into two alternating register sets.
-template <int FM_, int FN_, int NW_, int U_, int APF_ = 0>
+template <int FM_, int FN_, int NW_, int U_>
 struct SkinnyCfg {
-    static constexpr int FM = FM_, FN = FN_, NW = NW_, U = U_, APF = APF_;
+    static constexpr int FM = FM_, FN = FN_, NW = NW_, U = U_;
     static constexpr int THREADS = 64 * NW;
     static constexpr int MAX_M = 16 * FM, BN = 16 * FN;
     static constexpr int LDS_BYTES = FM * FN * 64 * 16;  // one block set: the waves add into it
@@ -90,32 +86,6 @@ gemm_skinny_kernel(const GemmArgs p)
             for (int j = 0; j < FN; ++j) acc[i][j] = mfma16(bod[j], aod, acc[i][j]);
         }
     };
-    if constexpr (Cfg::APF) {
-        for (int c0 = wave * U; c0 < nchunks; c0 += NW * U) {
-            v4i bq[U][FN], aq[2][FM];
-            auto load_a = [&](int u, v4i (&dst)[FM]) __attribute__((always_inline)) {
-                const int kofs = (c0 + u) * 64;
-                const bool ok = kofs + ld_ch * 16 < Kb;
-#pragma unroll
-                for (int i = 0; i < FM; ++i)
-                    dst[i] = ok ? *reinterpret_cast<const v4i *>(p.A + a_off[i] + kofs) : v4i{0, 0, 0, 0};
-            };
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int kofs = (c0 + u) * 64;
-                const bool ok = kofs + ld_ch * 16 < Kb;  // also false for c0+u >= nchunks
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    bq[u][j] = ok ? __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p.B + b_off[j] + kofs)) : v4i{0, 0, 0, 0};
-            }
-            load_a(0, aq[0]);
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (u + 1 < U) load_a(u + 1, aq[(u + 1) & 1]);
-                contract(bq[u], aq[u & 1]);
-            }
-        }
-    } else
     for (int c0 = wave * U; c0 < nchunks; c0 += NW * U) {
         v4i bq[U][FN], aq[U][FM];
 #pragma unroll

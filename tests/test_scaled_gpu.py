@@ -87,8 +87,8 @@ def test_rejections():
     a = torch.zeros((m, k // 2), dtype=torch.int8, device=DEV)
     d = torch.zeros((m, n), dtype=torch.float16, device=DEV)
     names = qm.config_names()
-    with pytest.raises(qm.QuadmulError):  # the eight-wave variant has no scaled output (its registers do not hold the scales)
-        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q256x256_w2x4_s4o1"))
+    with pytest.raises(qm.QuadmulError):  # the 256 x 128 tile two to a CU has no scaled output (its registers do not hold the scales)
+        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q256x128_w2x2_s3o2"))
     with pytest.raises(qm.QuadmulError):  # partial sums cannot meet in a rounded output: a K split needs a workspace
         qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s4o1") | (2 << 24), workspace=None)
     with pytest.raises(qm.QuadmulError):
