@@ -777,6 +777,20 @@ static hipError_t launch_split_with_workspace(GemmArgs p, const Choice &ch, void
     return hipGetLastError();
 }
 
+// An A of 2 GiB or more is beyond the 32-bit row offsets of the fast kernels; its row blocks
+// are independent (block r0.. of A gives rows r0.. of C), so the call is cut into blocks
+// of rows that fit, one after the other on the stream (they share the workspace).  Returns
+// the rows per block, 0 when the call needs no cutting or cutting does not help (B too large
+// as well, or a shape the fast kernels do not take anyway).
+static int row_block_for_large_a(int m, int n, int k, int ptr_align)
+{
+    if (k < 32 || k % 32 != 0 || k > QM_MAX_K_X16 || ptr_align < 16) return 0;
+    const long long kb = k / 2;
+    if ((long long)m * kb < 0x7fffffffLL || (long long)n * kb >= 0x7fffffffLL) return 0;
+    const long long rows = ((0x7fffffffLL - 1) / kb) & ~255LL;
+    return rows >= 256 ? (int)rows : 0;
+}
+
 }  // namespace qm
 
 using namespace qm;
@@ -795,6 +809,15 @@ QM_EXPORT int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n,
         return e == hipSuccess ? QM_OK : fail_launch(e);
     }
     const int align = ptr_alignment(A, B);
+    if (const int rb = cfg == QM_CFG_AUTO ? row_block_for_large_a(m, n, k, align) : 0) {
+        for (int r0 = 0; r0 < m; r0 += rb) {
+            const int st_b = qm_gemm_i4_ws(static_cast<const uint8_t *>(A) + (size_t)r0 * (size_t)(k / 2), B,
+                                           static_cast<int32_t *>(C) + (size_t)r0 * (size_t)n, m - r0 < rb ? m - r0 : rb, n, k,
+                                           stream, cfg, workspace, workspace_bytes);
+            if (st_b != QM_OK) return st_b;
+        }
+        return QM_OK;
+    }
     const bool has_ws = workspace != nullptr && workspace_bytes > 0;
     Choice ch;
     if (cfg == QM_CFG_AUTO) {
@@ -852,6 +875,16 @@ QM_EXPORT int qm_gemm_i4_scaled_ws(const void *A, const void *B, void *D, int m,
         return e == hipSuccess ? QM_OK : fail_launch(e);
     }
     const int align = ptr_alignment(A, B);
+    if (const int rb = cfg == QM_CFG_AUTO ? row_block_for_large_a(m, n, k, align) : 0) {
+        for (int r0 = 0; r0 < m; r0 += rb) {
+            const int st_b = qm_gemm_i4_scaled_ws(static_cast<const uint8_t *>(A) + (size_t)r0 * (size_t)(k / 2), B,
+                                                  static_cast<uint16_t *>(D) + (size_t)r0 * (size_t)n, m - r0 < rb ? m - r0 : rb, n,
+                                                  k, row_scale ? row_scale + r0 : nullptr, col_scale, out_dtype, stream, cfg,
+                                                  workspace, workspace_bytes);
+            if (st_b != QM_OK) return st_b;
+        }
+        return QM_OK;
+    }
     const bool has_ws = workspace != nullptr && workspace_bytes > 0;
     GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(D), m, n, k};
     p.row_scale = row_scale;
@@ -911,6 +944,12 @@ QM_EXPORT int qm_gemm_i4_scaled(const void *A, const void *B, void *D, int m, in
 QM_EXPORT size_t qm_gemm_workspace_bytes(int m, int n, int k, int ptr_align, int cfg, int scaled)
 {
     if (m < 1 || n < 1 || k < 2 || (k & 1)) return 0;
+    if (const int rb = cfg == QM_CFG_AUTO ? row_block_for_large_a(m, n, k, ptr_align) : 0) {
+        // the blocks run one after the other: the largest need of the two block sizes
+        const size_t whole = qm_gemm_workspace_bytes(rb, n, k, ptr_align, cfg, scaled);
+        const size_t rest = m % rb ? qm_gemm_workspace_bytes(m % rb, n, k, ptr_align, cfg, scaled) : 0;
+        return whole > rest ? whole : rest;
+    }
     Choice ch;
     if (cfg == QM_CFG_AUTO) {
         ch = scaled ? select_scaled(m, n, k, ptr_align, true) : select_config(m, n, k, ptr_align, true);

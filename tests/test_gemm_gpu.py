@@ -517,3 +517,58 @@ def test_short_last_k_step_on_every_pipelined_config(oracle_mod, k):
         assert (run_gemm(hi_a, lo_b, m, n, k, cfg) == -56 * k).all(), name   # every nibble counted exactly once
         ran += 1
     assert ran >= 8
+
+
+def test_operands_of_two_gib_and_more(oracle_mod):
+    """An A of 2 GiB or more is cut into row blocks that fit the fast kernels' 32-bit row
+    offsets; a B that large goes to the generic kernel (64-bit offsets).  Every row is compared
+    with the library's own result on slices below the limit (paths the other tests pin against
+    the oracle), and the rows either side of the block boundary and the last rows with the
+    oracle itself.  Packed bytes are drawn on the GPU: any byte is two valid nibbles."""
+    import quadmul
+
+    k, kb = 4096, 2048
+    g = torch.Generator(device=DEV).manual_seed(SEED_BASE + 6100)
+    # --- large A ---
+    m, n = (1 << 20) + 300, 48
+    assert m * kb >= 2 ** 31
+    a_d = torch.randint(-128, 128, (m, kb), dtype=torch.int8, device=DEV, generator=g)
+    b_d = torch.randint(-128, 128, (n, kb), dtype=torch.int8, device=DEV, generator=g)
+    want = torch.empty((m, n), dtype=torch.int32, device=DEV)
+    for r0 in range(0, m, 65536):
+        rows = min(65536, m - r0)
+        qm.gemm(a_d[r0:r0 + rows], b_d, want[r0:r0 + rows], rows, n, k)
+    block = ((2 ** 31 - 2) // kb) & ~255
+    assert 0 < block < m
+    for fn in (lambda c: quadmul.gemm(a_d, b_d, c, m, n, k), lambda c: qm.gemm(a_d, b_d, c, m, n, k, workspace=None)):
+        c_d = poisoned_c(m, n, DEV)
+        fn(c_d)
+        torch.cuda.synchronize()
+        assert torch.equal(c_d, want)
+    for r0 in (0, block - 24, m - 40):
+        ref = oracle_mod.gemm_i4(a_d[r0:r0 + 40].cpu().numpy(), b_d.cpu().numpy())
+        assert oracle_mod.compare(c_d[r0:r0 + 40].cpu().numpy(), ref) == -1
+    # the scaled output takes the same road, with the row scales of each block
+    rs = torch.rand(m, device=DEV, generator=g) * 0.01 + 0.001
+    cs = torch.rand(n, device=DEV, generator=g) + 0.5
+    d_d = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+    quadmul.gemm_scaled(a_d, b_d, d_d, m, n, k, rs, cs)
+    torch.cuda.synchronize()
+    for r0 in (0, block - 24, m - 40):
+        ref = oracle_mod.scale_round16(want[r0:r0 + 40].cpu().numpy(), rs[r0:r0 + 40].cpu().numpy(), cs.cpu().numpy(), oracle_mod.OUT_F16)
+        assert np.array_equal(d_d[r0:r0 + 40].cpu().numpy().view(np.uint16), ref)
+    del a_d, want, c_d, d_d
+    # --- large B ---
+    m, n = 8, (1 << 20) + 20
+    a_d = torch.randint(-128, 128, (m, kb), dtype=torch.int8, device=DEV, generator=g)
+    b_d = torch.randint(-128, 128, (n, kb), dtype=torch.int8, device=DEV, generator=g)
+    assert qm.config_name(qm.select_config(m, n, k) & 0xFFFF) == "generic"
+    c_d = poisoned_c(m, n, DEV)
+    quadmul.gemm(a_d, b_d, c_d, m, n, k)
+    for c0 in range(0, n, 262144):
+        cols = min(262144, n - c0)
+        part = torch.empty((m, cols), dtype=torch.int32, device=DEV)
+        qm.gemm(a_d, b_d[c0:c0 + cols], part, m, cols, k)
+        assert torch.equal(c_d[:, c0:c0 + cols], part)
+    ref = oracle_mod.gemm_i4(a_d.cpu().numpy(), b_d[n - 50:].cpu().numpy())
+    assert oracle_mod.compare(np.ascontiguousarray(c_d[:, n - 50:].cpu().numpy()), ref) == -1
