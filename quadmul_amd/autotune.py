@@ -152,7 +152,7 @@ def emit_table(tuned: List[Dict], path: str) -> None:
         "// Per-shape kernel choice measured on MI355X: {M, N, K, \"config name\", group_m, ksplit,",
         "// one item per workgroup}.",
         "// Written by quadmul_amd/autotune.py; shapes not listed use the cost model in",
-        "// qm_dispatch.hip.  Counterpart of the reference's A40 table (configs.cu:19-689).",
+        "// qm_select.hpp.  Counterpart of the reference's A40 table (configs.cu:19-689).",
     ]
     for t in tuned:
         b = t["best"]

@@ -11,396 +11,14 @@
 #include "../../include/qm_abi.h"
 #include "qm_launch.hpp"
 #include "qm_skinny.hpp"
+#include "qm_aux.hpp"
 
 #define QM_EXPORT extern "C" __attribute__((visibility("default")))
 
 namespace qm {
 
 // --------------------------------------------------------------------------
-// Fallback kernel: any M, N, even K, any alignment, no limit on K.  One thread
-// per element of C over LDS-staged 16x16x(128 nibble) tiles, plain byte loads.
-// --------------------------------------------------------------------------
-__device__ __forceinline__ int s4_lo(uint32_t b) { return (int)(int8_t)(b << 4) >> 4; }
-__device__ __forceinline__ int s4_hi(uint32_t b) { return (int)(int8_t)b >> 4; }
-
-__global__ void __launch_bounds__(256) gemm_generic_kernel(const GemmArgs p, const int tiles_n)
-{
-    __shared__ uint8_t As[16][64 + 4];
-    __shared__ uint8_t Bs[16][64 + 4];
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    const int m0 = (blockIdx.x / tiles_n) * 16, n0 = (blockIdx.x % tiles_n) * 16;
-    const size_t Kb = (size_t)(p.K >> 1);
-    int32_t sum = 0;
-    for (size_t k0 = 0; k0 < Kb; k0 += 64) {
-        // 16 rows x 64 bytes per operand = 1024 bytes each, 4 bytes per thread
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const int idx = threadIdx.x + t * 256, row = idx >> 6, col = idx & 63;
-            const bool kin = k0 + col < Kb;
-            As[row][col] = (kin && m0 + row < p.M) ? p.A[(size_t)(m0 + row) * Kb + k0 + col] : (uint8_t)0;
-            Bs[row][col] = (kin && n0 + row < p.N) ? p.B[(size_t)(n0 + row) * Kb + k0 + col] : (uint8_t)0;
-        }
-        __syncthreads();
-#pragma unroll 16
-        for (int j = 0; j < 64; ++j) {
-            const uint32_t a = As[ty][j], b = Bs[tx][j];
-            sum += s4_lo(a) * s4_lo(b) + s4_hi(a) * s4_hi(b);
-        }
-        __syncthreads();
-    }
-    const int m = m0 + ty, n = n0 + tx;
-    if (m < p.M && n < p.N) {
-        const size_t at = (size_t)m * p.N + n;
-        if (p.out == OUT_I32) p.C[at] = sum;
-        else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(sum, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
-    }
-}
-
-static hipError_t launch_generic(const GemmArgs &p, hipStream_t stream, int)
-{
-    const long long tiles_m = (p.M + 15) / 16, tiles_n = (p.N + 15) / 16;
-    if (tiles_m * tiles_n > 0x7fffffffLL) return hipErrorInvalidValue;
-    gemm_generic_kernel<<<dim3((unsigned)(tiles_m * tiles_n)), dim3(256), 0, stream>>>(p, (int)tiles_n);
-    return hipGetLastError();
-}
-
-// --------------------------------------------------------------------------
-// Zero fill (k == 0) and pack / unpack, flat over the whole array: K is even so
-// a byte never straddles two rows.
-// --------------------------------------------------------------------------
-__global__ void fill_zero16_kernel(uint16_t *dst, size_t n)
-{
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = 0;
-}
-
-__global__ void fill_zero_kernel(int32_t *dst, size_t n)
-{
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = 0;
-}
-
-// --------------------------------------------------------------------------
-// Operand copy with every row padded with zeros to a whole number of 128-nibble K-steps
-// (zero nibbles add nothing to a product): what lets the pipelined kernel run shapes whose
-// K is not a multiple of 128, or whose operands are not 16-byte aligned, out of a
-// caller-provided workspace.  kb / kbp: bytes per row of the source / of the copy.
-// --------------------------------------------------------------------------
-__global__ void pad_rows_vec_kernel(const v4i *__restrict__ src, v4i *__restrict__ dst, int rows, int kb16, int kbp16)
-{
-    const size_t total = (size_t)rows * kbp16;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const size_t r = i / kbp16;
-        const int c = (int)(i - r * kbp16);
-        dst[i] = c < kb16 ? src[r * kb16 + c] : v4i{0, 0, 0, 0};
-    }
-}
-
-__global__ void pad_rows_byte_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int rows, int kb, int kbp)
-{
-    const size_t total = (size_t)rows * kbp;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const size_t r = i / kbp;
-        const int c = (int)(i - r * kbp);
-        dst[i] = c < kb ? src[r * kb + c] : (uint8_t)0;
-    }
-}
-
-// --------------------------------------------------------------------------
-// K split with a workspace (pipelined kernel): item (split s, tile t) of the GEMM launch
-// left its BM x BN partial sums in slot s * ntiles + t, wave by wave, block by block, 16
-// bytes per lane in the order the MFMA leaves a block (lane l: row l % 16, columns
-// 4 * (l / 16) .. + 3).  One thread here adds up the splits of one such 16-byte piece and
-// stores the four sums -- as int32, or scaled and rounded to a 16-bit float -- with the
-// guards of the matrix edge.  Tiles are numbered as the GEMM kernel numbers them (columns of
-// group_m tiles).
-// --------------------------------------------------------------------------
-struct SplitReduceArgs {
-    const v4i *ws;
-    void *C;
-    int M, N;
-    int tiles_m, tiles_n, group_m, ksplit;
-    int BM, BN, WGN, FM, FN, waves;
-    const float *row_scale, *col_scale;
-    int out;
-};
-
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitReduceArgs q)
-{
-    const int blocks = q.FM * q.FN;
-    const size_t per_tile = (size_t)q.waves * blocks * 64;  // 16-byte pieces per slot
-    const size_t ntiles = (size_t)q.tiles_m * q.tiles_n;
-    const uint32_t t = blockIdx.x * 256u + threadIdx.x;  // (the launcher keeps the count below 2^31)
-    if (t >= ntiles * per_tile) return;
-    const v4i *src = q.ws + t;
-    const size_t stride = ntiles * per_tile;
-    v4i sum = {0, 0, 0, 0};
-    // four splits at a time, so that their loads are in flight together (splits past the
-    // last re-read it and count for nothing)
-    for (int s = 0; s < q.ksplit; s += 4) {
-        v4i v[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = __builtin_nontemporal_load(src + (size_t)min(s + i, q.ksplit - 1) * stride);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int on = s + i < q.ksplit ? -1 : 0;
-            sum.x += v[i].x & on; sum.y += v[i].y & on; sum.z += v[i].z & on; sum.w += v[i].w & on;
-        }
-    }
-    const int lane = (int)(t & 63);
-    uint32_t u = t >> 6;
-    const int blk = (int)(u % (uint32_t)blocks);
-    u /= (uint32_t)blocks;
-    const int wave = (int)(u % (uint32_t)q.waves);
-    const int pid = (int)(u / (uint32_t)q.waves);
-    const int width = q.group_m * q.tiles_n;
-    const int first_m = (pid / width) * q.group_m;
-    const int gsz = min(q.tiles_m - first_m, q.group_m);
-    const int tm = first_m + (pid % width) % gsz, tn = (pid % width) / gsz;
-    const int m = tm * q.BM + (wave / q.WGN) * q.FM * 16 + (blk / q.FN) * 16 + (lane & 15);
-    const int n = tn * q.BN + (wave % q.WGN) * q.FN * 16 + (blk % q.FN) * 16 + (lane >> 4) * 4;
-    if (m >= q.M || n >= q.N) return;
-    if (q.out == OUT_I32) {
-        int32_t *crow = static_cast<int32_t *>(q.C) + (size_t)m * q.N;
-        if ((q.N & 3) == 0 && ((uintptr_t)q.C & 15) == 0) {
-            *reinterpret_cast<v4i *>(crow + n) = sum;  // n % 4 == 0 and N % 4 == 0: all four inside
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (n + e < q.N) crow[n + e] = sum[e];
-        }
-    } else {
-        uint16_t *drow = static_cast<uint16_t *>(q.C) + (size_t)m * q.N;
-        const float rs = scale_at(q.row_scale, m, q.M);
-        uint16_t h[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int c = sum[e];
-            h[e] = round16(scaled(c, rs, scale_at(q.col_scale, n + e, q.N)), q.out);
-        }
-        if ((q.N & 3) == 0 && ((uintptr_t)q.C & 7) == 0) {
-            *reinterpret_cast<v2i *>(drow + n) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (n + e < q.N) drow[n + e] = h[e];
-        }
-    }
-}
-
-// 16 int8 in -> 8 packed bytes out per thread when aligned, else one byte per thread.
-__device__ __forceinline__ uint32_t pack4(uint32_t w)  // 4 int8 -> 2 packed bytes in bits 0..15
-{
-    uint32_t t = w & 0x0F0F0F0Fu;
-    t |= t >> 4;  // byte0 = n0 | n1<<4, byte2 = n2 | n3<<4
-    return (t & 0xFFu) | ((t >> 8) & 0xFF00u);
-}
-
-__global__ void pack_i4_vec_kernel(const v4i *__restrict__ src, v2i *__restrict__ dst, size_t nvec)
-{
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (size_t)gridDim.x * blockDim.x) {
-        const v4i v = src[i];
-        v2i o;
-        o.x = (int)(pack4((uint32_t)v.x) | (pack4((uint32_t)v.y) << 16));
-        o.y = (int)(pack4((uint32_t)v.z) | (pack4((uint32_t)v.w) << 16));
-        dst[i] = o;
-    }
-}
-
-__global__ void pack_i4_byte_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, size_t nbytes)
-{
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nbytes; i += (size_t)gridDim.x * blockDim.x)
-        dst[i] = (uint8_t)((src[2 * i] & 0x0Fu) | ((src[2 * i + 1] & 0x0Fu) << 4));
-}
-
-// 4 packed bytes -> 8 int8: widen nibbles to bytes, sign-extend (bit 3 set => OR 0xF0),
-// interleave even/odd elements back into K order.
-__device__ __forceinline__ uint32_t sext_nibbles(uint32_t x)  // x = 0x0n0n0n0n
-{
-    const uint32_t t = x & 0x08080808u;
-    return x | ((t << 5) - (t << 1));  // 0x08 -> 0xF0 in each byte (the top byte wraps mod 2^32)
-}
-
-__global__ void unpack_i4_vec_kernel(const uint32_t *__restrict__ src, v2i *__restrict__ dst, size_t nwords)
-{
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nwords; i += (size_t)gridDim.x * blockDim.x) {
-        const uint32_t w = src[i];
-        const uint32_t ev = sext_nibbles(w & 0x0F0F0F0Fu), od = sext_nibbles((w >> 4) & 0x0F0F0F0Fu);
-        v2i o;  // bytes: ev0 od0 ev1 od1 | ev2 od2 ev3 od3
-        o.x = (int)__builtin_amdgcn_perm(od, ev, 0x05010400u);
-        o.y = (int)__builtin_amdgcn_perm(od, ev, 0x07030602u);
-        dst[i] = o;
-    }
-}
-
-__global__ void unpack_i4_byte_kernel(const uint8_t *__restrict__ src, int8_t *__restrict__ dst, size_t nbytes)
-{
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nbytes; i += (size_t)gridDim.x * blockDim.x) {
-        const uint32_t b = src[i];
-        dst[2 * i] = (int8_t)s4_lo(b);
-        dst[2 * i + 1] = (int8_t)s4_hi(b);
-    }
-}
-
-// --------------------------------------------------------------------------
-// Per-row symmetric quantisation to int4 fused with the packing: one workgroup per row,
-// the row held in registers between the two passes over it (maximum, then quantise), so
-// HBM is read once.  x is fp16, bf16 or fp32; 8 elements (4 packed bytes) per thread-chunk.
-// --------------------------------------------------------------------------
-template <int IN> struct QuantIn;
-template <> struct QuantIn<QM_IN_F16> {
-    static constexpr int BYTES = 2;
-    static __device__ __forceinline__ float widen(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
-};
-template <> struct QuantIn<QM_IN_BF16> {
-    static constexpr int BYTES = 2;
-    static __device__ __forceinline__ float widen(uint16_t h) { return __builtin_bit_cast(float, (uint32_t)h << 16); }
-};
-template <> struct QuantIn<QM_IN_F32> {
-    static constexpr int BYTES = 4;
-};
-
-template <int IN>
-__device__ __forceinline__ void load8(const uint8_t *src, float (&v)[8])
-{
-    if constexpr (IN == QM_IN_F32) {
-        const v4i lo = *reinterpret_cast<const v4i *>(src), hi = *reinterpret_cast<const v4i *>(src + 16);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int a = lo[e], b = hi[e];
-            v[e] = __builtin_bit_cast(float, a);
-            v[4 + e] = __builtin_bit_cast(float, b);
-        }
-    } else {
-        const v4i w = *reinterpret_cast<const v4i *>(src);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint32_t d = (uint32_t)w[e];
-            v[2 * e] = QuantIn<IN>::widen((uint16_t)(d & 0xFFFFu));
-            v[2 * e + 1] = QuantIn<IN>::widen((uint16_t)(d >> 16));
-        }
-    }
-}
-
-__device__ __forceinline__ uint32_t quant8(const float (&v)[8], float inv)
-{
-#pragma clang fp contract(off)
-    uint32_t out = 0;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        float r = __builtin_rintf(v[e] * inv);  // round half to even
-        r = fminf(fmaxf(r, -7.0f), 7.0f);
-        out |= ((uint32_t)(int)r & 0xFu) << (4 * e);  // element e -> nibble e: low nibble = even k (test.py:8,14)
-    }
-    return out;
-}
-
-// workgroup-wide maximum of non-negative floats
-__device__ __forceinline__ float block_max(float x, float *lds)
-{
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) x = fmaxf(x, __shfl_xor(x, off));
-    const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) lds[wave] = x;
-    __syncthreads();
-    float m = lds[0];
-    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) m = fmaxf(m, lds[w]);
-    __syncthreads();
-    return m;
-}
-
-// NC: chunks of 8 elements a thread keeps in registers (k <= 2048 * NC); NC == 0: any k that is
-// a multiple of 8, the row read twice (the second time out of the L2)
-template <int IN, int NC>
-__global__ void __launch_bounds__(256) quantize_pack_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ dst, float *__restrict__ scales, int k)
-{
-    __shared__ float red[4];
-    const int row = blockIdx.x, tid = threadIdx.x, nchunks = k >> 3;
-    const uint8_t *xr = x + (size_t)row * k * QuantIn<IN>::BYTES;
-    uint32_t *out = reinterpret_cast<uint32_t *>(dst + (size_t)row * (k >> 1));
-    float amax = 0.0f;
-    if constexpr (NC > 0) {
-        float v[NC][8];
-#pragma unroll
-        for (int i = 0; i < NC; ++i) {
-            const int c = tid + i * 256;
-            if (c < nchunks) {
-                load8<IN>(xr + (size_t)c * 8 * QuantIn<IN>::BYTES, v[i]);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[i][e]));
-            }
-        }
-        amax = block_max(amax, red);
-        const float inv = amax > 0.0f ? 7.0f / amax : 0.0f;
-        if (tid == 0) scales[row] = amax / 7.0f;
-#pragma unroll
-        for (int i = 0; i < NC; ++i) {
-            const int c = tid + i * 256;
-            if (c < nchunks) out[c] = quant8(v[i], inv);
-        }
-    } else {
-        float v[8];
-        for (int c = tid; c < nchunks; c += 256) {
-            load8<IN>(xr + (size_t)c * 8 * QuantIn<IN>::BYTES, v);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) amax = fmaxf(amax, fabsf(v[e]));
-        }
-        amax = block_max(amax, red);
-        const float inv = amax > 0.0f ? 7.0f / amax : 0.0f;
-        if (tid == 0) scales[row] = amax / 7.0f;
-        for (int c = tid; c < nchunks; c += 256) {
-            load8<IN>(xr + (size_t)c * 8 * QuantIn<IN>::BYTES, v);
-            out[c] = quant8(v, inv);
-        }
-    }
-}
-
-// any even k, any alignment: one pair of elements per thread and pass
-template <int IN>
-__global__ void __launch_bounds__(256) quantize_pack_scalar_kernel(const uint8_t *__restrict__ x, uint8_t *__restrict__ dst, float *__restrict__ scales, int k)
-{
-#pragma clang fp contract(off)
-    __shared__ float red[4];
-    const int row = blockIdx.x, tid = threadIdx.x;
-    auto at = [&](int j) -> float {
-        if constexpr (IN == QM_IN_F32) {
-            return reinterpret_cast<const float *>(x)[(size_t)row * k + j];
-        } else {
-            return QuantIn<IN>::widen(reinterpret_cast<const uint16_t *>(x)[(size_t)row * k + j]);
-        }
-    };
-    float amax = 0.0f;
-    for (int j = tid; j < k; j += 256) amax = fmaxf(amax, fabsf(at(j)));
-    amax = block_max(amax, red);
-    const float inv = amax > 0.0f ? 7.0f / amax : 0.0f;
-    if (tid == 0) scales[row] = amax / 7.0f;
-    for (int j = 2 * tid; j < k; j += 512) {
-        const float r0 = fminf(fmaxf(__builtin_rintf(at(j) * inv), -7.0f), 7.0f), r1 = fminf(fmaxf(__builtin_rintf(at(j + 1) * inv), -7.0f), 7.0f);
-        dst[(size_t)row * (k >> 1) + (j >> 1)] = (uint8_t)(((int)r0 & 0xF) | (((int)r1 & 0xF) << 4));
-    }
-}
-
-template <int IN>
-static hipError_t launch_quantize_pack(const void *x, void *dst, float *scales, int rows, int k, hipStream_t s)
-{
-    const uint8_t *xb = static_cast<const uint8_t *>(x);
-    uint8_t *db = static_cast<uint8_t *>(dst);
-    const bool vec = k % 8 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)dst & 3) == 0;
-    if (!vec) quantize_pack_scalar_kernel<IN><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
-    else if (k <= 2048 * 2) quantize_pack_kernel<IN, 2><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
-    else if (k <= 2048 * 8) quantize_pack_kernel<IN, 8><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
-    else quantize_pack_kernel<IN, 0><<<dim3(rows), dim3(256), 0, s>>>(xb, db, scales, k);
-    return hipGetLastError();
-}
-
-static unsigned flat_grid(size_t items, unsigned block)
-{
-    size_t g = (items + block - 1) / block;
-    if (g < 1) g = 1;
-    if (g > 256u * 32u) g = 256u * 32u;
-    return (unsigned)g;
-}
-
-// --------------------------------------------------------------------------
-// Skinny launchers
+// Launchers of the skinny and dot kernels
 // --------------------------------------------------------------------------
 template <class Cfg>
 static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
@@ -422,210 +40,11 @@ static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int)
     hipError_t QM_DOT_FN(MR, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_dot<DotCfg<MR, FN, NW, U>>(p, s, gm); }
 #include "qm_configs.inc"
 
-// --------------------------------------------------------------------------
-// Configuration registry
-// --------------------------------------------------------------------------
-enum Kind { KIND_GENERIC = 0, KIND_SKINNY = 2, KIND_TILE16 = 3 };
+}  // namespace qm
 
-struct ConfigDesc {
-    const char *name;
-    int kind;
-    int bm, bn, bk;  // tile: block shape; skinny: bm = max M, bn = columns per workgroup
-    int waves, mode;
-    LaunchFn launch;
-    int wgm = 0, wgn = 0;  // pipelined kernel: waves down and across the tile
-};
+#include "qm_select.hpp"
 
-#define QM_STR2(x) #x
-#define QM_STR(x) QM_STR2(x)
-static const ConfigDesc g_configs[] = {
-    {"generic", KIND_GENERIC, 16, 16, 128, 4, 0, &launch_generic},
-#define QM_TILE16(tu, BM, BN, WGM, WGN, ST, OCC)                                                              \
-    {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_s" QM_STR(ST) "o" QM_STR(OCC), KIND_TILE16, BM, BN, 128, \
-     (WGM) * (WGN), 0, &QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC), WGM, WGN},
-#define QM_SKINNY(FM, FN, NW, U)                                                     \
-    {"s" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
-     &QM_SKINNY_FN(FM, FN, NW, U)},
-#define QM_DOT(MR, FN, NW, U)                                                     \
-    {"v" QM_STR(MR) "x" QM_STR(FN) "_w" QM_STR(NW) "_u" QM_STR(U), KIND_SKINNY, MR, 16 * (FN), 128, NW, 0, \
-     &QM_DOT_FN(MR, FN, NW, U)},
-#include "qm_configs.inc"
-};
-static constexpr int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
-
-// Pipelined configurations that also exist with the scaled 16-bit float output
-static const struct { const char *name; LaunchFn launch; } g_scaled_tile16[] = {
-#define QM_TILE16S(tu, BM, BN, WGM, WGN, ST, OCC) \
-    {"q" QM_STR(BM) "x" QM_STR(BN) "_w" QM_STR(WGM) "x" QM_STR(WGN) "_s" QM_STR(ST) "o" QM_STR(OCC), &QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC)},
-#include "qm_configs.inc"
-};
-
-// The launcher of configuration cfg for the scaled output, or null: the generic and the
-// skinny kernels take the output form at run time, the pipelined ones as separate kernels
-// (not every configuration has them).
-static LaunchFn scaled_launcher(int cfg)
-{
-    const ConfigDesc &c = g_configs[cfg];
-    if (c.kind == KIND_GENERIC || c.kind == KIND_SKINNY) return c.launch;
-    if (c.kind == KIND_TILE16)
-        for (const auto &e : g_scaled_tile16)
-            if (std::strcmp(e.name, c.name) == 0) return e.launch;
-    return nullptr;
-}
-
-static int find_config(const char *name)
-{
-    for (int i = 0; i < g_num_configs; ++i)
-        if (std::strcmp(g_configs[i].name, name) == 0) return i;
-    return -1;
-}
-
-// The 16-byte-load kernels need whole, aligned chunks and 32-bit row offsets,
-// and the x16 widening bounds K.
-static bool fast_path_ok(int m, int n, int k, int ptr_align)
-{
-    if (k % 32 != 0 || k > QM_MAX_K_X16 || ptr_align < 16) return false;
-    const long long kb = k / 2;
-    return (long long)m * kb < 0x7fffffffLL && (long long)n * kb < 0x7fffffffLL;
-}
-
-static bool config_supports(int cfg, int m, int n, int k, int ptr_align)
-{
-    if (cfg < 0 || cfg >= g_num_configs || m < 1 || n < 1 || k < 2 || (k & 1)) return false;
-    const ConfigDesc &c = g_configs[cfg];
-    if (c.kind == KIND_GENERIC) return true;
-    if (!fast_path_ok(m, n, k, ptr_align)) return false;
-    if (c.kind == KIND_SKINNY) return m <= c.bm;
-    if (c.kind == KIND_TILE16) return k % 128 == 0 || k > 128;  // a short last K-step needs a step before it
-    return true;
-}
-
-// --------------------------------------------------------------------------
-// Shape table (autotuned on MI355X; regenerated by quadmul_amd/autotune.py) with
-// a cost-model fallback -- the reference instead skips unknown shapes.
-// --------------------------------------------------------------------------
-struct TableEntry {
-    int m, n, k;
-    const char *config;
-    int group_m, ksplit;
-    int spread;  // 1: one work item per workgroup instead of a persistent grid (pipelined kernel)
-};
-static const TableEntry g_table[] = {
-#include "qm_tile_table.inc"
-    {0, 0, 0, nullptr, 0, 0},
-};
-
-struct Choice {
-    int cfg, group_m, ksplit;
-    int spread = 0;
-};
-
-static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
-{
-    if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
-    if (m <= 2) {
-        const int id = find_config(m == 1 ? "v1x1_w8_u4" : "v2x1_w16_u2");
-        if (id >= 0) return {id, 1, 1};
-    }
-    if (m <= 64) {
-        const int fm = m <= 16 ? 1 : (m <= 32 ? 2 : 4);
-        const char *name = fm == 1 ? "s1x1_w8_u4" : (fm == 2 ? "s2x1_w8_u4" : "s4x1_w16_u1");
-        const int id = find_config(name);
-        if (id >= 0) return {id, 1, 1};
-    }
-    // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency),
-    // over the configurations that can run this K.  Efficiencies are measured ratios.
-    // eff: throughput per tile area relative to the 256 x 256 tile with the GPU full (measured)
-    static const struct { const char *name; double eff; } cands[] = {
-        {"q256x256_w2x2_s4o1", 1.00}, {"q256x128_w2x2_s4o1", 0.82}, {"q128x256_w2x2_s4o1", 0.82}, {"q128x128_w2x2_s4o1", 0.60},
-        {"q128x64_w2x2_s4o2", 0.46},  {"q64x128_w2x2_s4o2", 0.44},  {"q64x64_w2x2_s4o2", 0.37},
-    };
-    int best = 0, best_ks = 1;
-    double best_cost = 1e300;
-    for (const auto &c : cands) {
-        const int id = find_config(c.name);
-        if (id < 0 || !config_supports(id, m, n, k, ptr_align)) continue;
-        const ConfigDesc &d = g_configs[id];
-        const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
-        // Few tiles and a long K: the pipelined kernel can split K over several workgroups
-        // per tile.  With a workspace the partial sums cost a second kernel (about 8 us all
-        // told, measured); without one they meet in C through 4-byte atomics, which are slow
-        // enough that splitting only pays when each split keeps a long K of its own
-        // (measured: wins at K = 28672, loses at K = 8192).
-        // Cost in units of 16.5 ps (one K-step of the 256 x 256 tile = 65536): K-steps per
-        // item x tile area / efficiency, plus 4 us per round of workgroups for filling the
-        // ring and writing out, plus the split's own cost.
-        const int kt = (k + 127) / 128;
-        auto cost_of = [&](int ks_) {
-            const double rounds = (double)((tiles * ks_ + 255) / 256);
-            return rounds * ((double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + 240000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
-        };
-        int ks = 1;
-        double cost = cost_of(1);
-        if (d.kind == KIND_TILE16 && has_ws) {
-            for (int t = 2; t <= 16 && tiles * t <= 256 && kt / t >= 4; ++t)
-                if (cost_of(t) < cost) { cost = cost_of(t); ks = t; }
-        } else if (d.kind == KIND_TILE16) {
-            while (ks < 4 && tiles * ks * 2 <= 256 && (k / 128) / (ks * 2) >= 48) ks *= 2;
-            if (ks > 1) cost = (double)d.bm * d.bn / c.eff * ((kt + ks - 1) / ks) * 1.25 + 180000.0;
-        }
-        if (cost < best_cost) { best_cost = cost; best = id; best_ks = ks; }
-    }
-    if (m <= 128) {
-        // 65..128 rows: the wave-level split-K kernel with eight row blocks has no ring to
-        // fill and no second kernel, and wins while N x K is small (measured: about 2 us
-        // plus 0.38 us per million elements of B, in the units above)
-        const int id = find_config("s8x1_w8_u1");
-        const double cost_s = (2.0 + (double)n * (double)k / 2.6e6) / 1.65e-5;
-        if (id >= 0 && cost_s < best_cost) return {id, 1, 1};
-    }
-    const int ksplit = best_ks;
-    return {best, 4, ksplit};
-}
-
-static Choice select_config(int m, int n, int k, int ptr_align, bool has_ws)
-{
-    static int resolved[sizeof(g_table) / sizeof(g_table[0])];
-    static std::once_flag once;
-    std::call_once(once, [] {
-        for (size_t i = 0; g_table[i].config; ++i) resolved[i] = find_config(g_table[i].config);
-    });
-    for (size_t i = 0; g_table[i].config; ++i)
-        if (g_table[i].m == m && g_table[i].n == n && g_table[i].k == k && resolved[i] >= 0 &&
-            config_supports(resolved[i], m, n, k, ptr_align))
-            return {resolved[i], g_table[i].group_m, g_table[i].ksplit > 0 ? g_table[i].ksplit : 1, g_table[i].spread};
-    return heuristic(m, n, k, ptr_align, has_ws);
-}
-
-// The scaled output has fewer kernels to choose from: the table's choice when that
-// configuration has the output form, else the best pipelined one that has it, else what the
-// heuristic says for skinny shapes, else the generic kernel.
-static Choice select_scaled(int m, int n, int k, int ptr_align, bool has_ws)
-{
-    const Choice ch = select_config(m, n, k, ptr_align, has_ws);
-    if (ch.ksplit <= 1 && scaled_launcher(ch.cfg)) return ch;
-    // K split: the int32 kernel of any pipelined configuration leaves partial sums in the
-    // workspace, and the kernel that adds them up scales and rounds
-    if (ch.ksplit > 1 && has_ws && g_configs[ch.cfg].kind == KIND_TILE16) return ch;
-    if (fast_path_ok(m, n, k, ptr_align) && k % 128 == 0) {
-        int best = -1;
-        double best_cost = 1e300;
-        for (const auto &e : g_scaled_tile16) {
-            const int id = find_config(e.name);
-            if (id < 0) continue;
-            const ConfigDesc &d = g_configs[id];
-            const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
-            const int area = d.bm * d.bn;
-            const double eff = area >= 256 * 256 ? 1.0 : (area >= 256 * 128 ? 0.82 : (area >= 128 * 128 ? 0.60 : (area >= 128 * 64 ? 0.45 : 0.37)));
-            const double cost = (double)((tiles + 255) / 256) * ((double)((k + 127) / 128) * area / eff + 240000.0);  // as in heuristic()
-            if (cost < best_cost) { best_cost = cost; best = id; }
-        }
-        if (best >= 0) return {best, 4, 1};
-    }
-    const Choice h = heuristic(m, n, k, ptr_align, false);
-    if (h.ksplit <= 1 && scaled_launcher(h.cfg)) return h;
-    return {0, 1, 1};
-}
+namespace qm {
 
 static thread_local int g_last_hip_error = 0;
 
@@ -791,6 +210,81 @@ static int row_block_for_large_a(int m, int n, int k, int ptr_align)
     return rows >= 256 ? (int)rows : 0;
 }
 
+// One GEMM call, arguments already checked (m, n >= 1, k even).  `out` is OUT_I32 with C in
+// `dst`, or OUT_F16 / OUT_BF16 with the scaled and rounded D there.  The two differ in one
+// place: a K split whose partial sums have no workspace to meet in falls back to atomic adds
+// into a zero-filled C for int32, and is not taken at all for a rounded output.
+static int run_gemm(const void *A, const void *B, void *dst, int m, int n, int k, const float *row_scale,
+                    const float *col_scale, int out, hipStream_t s, int cfg, void *workspace, size_t workspace_bytes)
+{
+    const bool scaled = out != OUT_I32;
+    const size_t cnt = (size_t)m * (size_t)n;
+    if (k == 0) {
+        if (scaled) fill_zero16_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<uint16_t *>(dst), cnt);
+        else fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(dst), cnt);
+        const hipError_t e = hipGetLastError();
+        return e == hipSuccess ? QM_OK : fail_launch(e);
+    }
+    const int align = ptr_alignment(A, B);
+    if (const int rb = cfg == QM_CFG_AUTO ? row_block_for_large_a(m, n, k, align) : 0) {
+        for (int r0 = 0; r0 < m; r0 += rb) {
+            const int st = run_gemm(static_cast<const uint8_t *>(A) + (size_t)r0 * (size_t)(k / 2), B,
+                                    static_cast<uint8_t *>(dst) + (size_t)r0 * (size_t)n * (scaled ? 2 : 4), m - r0 < rb ? m - r0 : rb,
+                                    n, k, row_scale ? row_scale + r0 : nullptr, col_scale, out, s, cfg, workspace, workspace_bytes);
+            if (st != QM_OK) return st;
+        }
+        return QM_OK;
+    }
+    const bool has_ws = workspace != nullptr && workspace_bytes > 0;
+    GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(dst), m, n, k};
+    p.row_scale = row_scale;
+    p.col_scale = col_scale;
+    p.out = out;
+    const auto launcher = [&](int id) { return scaled ? scaled_launcher(id) : g_configs[id].launch; };
+    Choice ch;
+    if (cfg == QM_CFG_AUTO) {
+        ch = scaled ? select_scaled(m, n, k, align, has_ws) : select_config(m, n, k, align, has_ws);
+    } else {
+        ch = choice_from_code(cfg);
+        if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
+        if (ch.ksplit > 1 && g_configs[ch.cfg].kind != KIND_TILE16) return QM_ERR_CONFIG;
+    }
+    ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
+    if (ch.ksplit > 1 && workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) {
+        const hipError_t e = launch_split_with_workspace(p, ch, workspace, s);
+        return e == hipSuccess ? QM_OK : fail_launch(e);
+    }
+    if (ch.ksplit > 1 && scaled) {
+        // partial sums cannot meet in a rounded output: without the workspace, no split
+        if (cfg != QM_CFG_AUTO) return QM_ERR_CONFIG;
+        ch = select_scaled(m, n, k, align, false);
+        ch.ksplit = 1;
+    }
+    if (cfg == QM_CFG_AUTO && has_ws) {
+        PadPlan pl = plan_padded_k(m, n, k, align, ch);
+        if (pl.on && !launcher(pl.ch.cfg)) {
+            // a pipelined configuration that has the scaled output, if the shape is one for those
+            const int id = find_config("q256x256_w2x2_s4o1");
+            if (id >= 0 && launcher(id)) pl.ch.cfg = id; else pl.on = false;
+        }
+        if (pl.on && ((uintptr_t)workspace & 15) == 0 && workspace_bytes >= pl.bytes()) {
+            hipError_t e = launch_padded(p, pl, workspace, s);
+            if (e == hipSuccess) e = launcher(pl.ch.cfg)(p, s, pl.ch.group_m | (1 << 8) | (pl.ch.spread << 16));
+            return e == hipSuccess ? QM_OK : fail_launch(e);
+        }
+    }
+    if (ch.ksplit > 1) {
+        // int32, no workspace: the partial sums meet in C by integer atomic adds, C starts from zero
+        fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(dst), cnt);
+        const hipError_t ez = hipGetLastError();
+        if (ez != hipSuccess) return fail_launch(ez);
+    }
+    const LaunchFn launch = launcher(ch.cfg);
+    if (!launch) return QM_ERR_CONFIG;
+    const hipError_t e = launch(p, s, ch.group_m | (ch.ksplit << 8) | (ch.spread << 16));
+    return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
 }  // namespace qm
 
 using namespace qm;
@@ -801,55 +295,7 @@ QM_EXPORT int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n,
     const int st = check_gemm_args(A, B, C, m, n, k);
     if (st != QM_OK) return st;
     if (m == 0 || n == 0) return QM_OK;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    if (k == 0) {
-        const size_t cnt = (size_t)m * (size_t)n;
-        fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(C), cnt);
-        const hipError_t e = hipGetLastError();
-        return e == hipSuccess ? QM_OK : fail_launch(e);
-    }
-    const int align = ptr_alignment(A, B);
-    if (const int rb = cfg == QM_CFG_AUTO ? row_block_for_large_a(m, n, k, align) : 0) {
-        for (int r0 = 0; r0 < m; r0 += rb) {
-            const int st_b = qm_gemm_i4_ws(static_cast<const uint8_t *>(A) + (size_t)r0 * (size_t)(k / 2), B,
-                                           static_cast<int32_t *>(C) + (size_t)r0 * (size_t)n, m - r0 < rb ? m - r0 : rb, n, k,
-                                           stream, cfg, workspace, workspace_bytes);
-            if (st_b != QM_OK) return st_b;
-        }
-        return QM_OK;
-    }
-    const bool has_ws = workspace != nullptr && workspace_bytes > 0;
-    Choice ch;
-    if (cfg == QM_CFG_AUTO) {
-        ch = select_config(m, n, k, align, has_ws);
-    } else {
-        ch = choice_from_code(cfg);
-        if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
-        if (ch.ksplit > 1 && g_configs[ch.cfg].kind != KIND_TILE16) return QM_ERR_CONFIG;
-    }
-    ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
-    GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(C), m, n, k};
-    if (cfg == QM_CFG_AUTO && has_ws) {
-        const PadPlan pl = plan_padded_k(m, n, k, align, ch);
-        if (pl.on && ((uintptr_t)workspace & 15) == 0 && workspace_bytes >= pl.bytes()) {
-            hipError_t e = launch_padded(p, pl, workspace, s);
-            if (e == hipSuccess) e = g_configs[pl.ch.cfg].launch(p, s, pl.ch.group_m | (1 << 8) | (pl.ch.spread << 16));
-            return e == hipSuccess ? QM_OK : fail_launch(e);
-        }
-    }
-    if (ch.ksplit > 1 && workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) {
-        const hipError_t e = launch_split_with_workspace(p, ch, workspace, s);
-        return e == hipSuccess ? QM_OK : fail_launch(e);
-    }
-    if (ch.ksplit > 1) {
-        // no workspace: split-K partial sums meet in C by integer atomic adds, C starts from zero
-        const size_t cnt = (size_t)m * (size_t)n;
-        fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(C), cnt);
-        const hipError_t ez = hipGetLastError();
-        if (ez != hipSuccess) return fail_launch(ez);
-    }
-    const hipError_t e = g_configs[ch.cfg].launch(p, s, ch.group_m | (ch.ksplit << 8) | (ch.spread << 16));
-    return e == hipSuccess ? QM_OK : fail_launch(e);
+    return run_gemm(A, B, C, m, n, k, nullptr, nullptr, OUT_I32, reinterpret_cast<hipStream_t>(stream), cfg, workspace, workspace_bytes);
 }
 
 QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg)
@@ -867,66 +313,8 @@ QM_EXPORT int qm_gemm_i4_scaled_ws(const void *A, const void *B, void *D, int m,
     if (!D) return QM_ERR_NULL;
     if ((uintptr_t)D & 1) return QM_ERR_ALIGN;
     if (k > 0 && (!A || !B)) return QM_ERR_NULL;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    if (k == 0) {
-        const size_t cnt = (size_t)m * (size_t)n;
-        fill_zero16_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<uint16_t *>(D), cnt);
-        const hipError_t e = hipGetLastError();
-        return e == hipSuccess ? QM_OK : fail_launch(e);
-    }
-    const int align = ptr_alignment(A, B);
-    if (const int rb = cfg == QM_CFG_AUTO ? row_block_for_large_a(m, n, k, align) : 0) {
-        for (int r0 = 0; r0 < m; r0 += rb) {
-            const int st_b = qm_gemm_i4_scaled_ws(static_cast<const uint8_t *>(A) + (size_t)r0 * (size_t)(k / 2), B,
-                                                  static_cast<uint16_t *>(D) + (size_t)r0 * (size_t)n, m - r0 < rb ? m - r0 : rb, n,
-                                                  k, row_scale ? row_scale + r0 : nullptr, col_scale, out_dtype, stream, cfg,
-                                                  workspace, workspace_bytes);
-            if (st_b != QM_OK) return st_b;
-        }
-        return QM_OK;
-    }
-    const bool has_ws = workspace != nullptr && workspace_bytes > 0;
-    GemmArgs p{static_cast<const uint8_t *>(A), static_cast<const uint8_t *>(B), static_cast<int32_t *>(D), m, n, k};
-    p.row_scale = row_scale;
-    p.col_scale = col_scale;
-    p.out = out_dtype == QM_OUT_F16 ? OUT_F16 : OUT_BF16;
-    Choice ch;
-    if (cfg == QM_CFG_AUTO) {
-        ch = select_scaled(m, n, k, align, has_ws);
-        ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
-        if (ch.ksplit > 1 && !workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) {
-            ch = select_scaled(m, n, k, align, false);  // too small a workspace: as without one
-            ch.ksplit = 1;
-        }
-    } else {
-        ch = choice_from_code(cfg);
-        if (!config_supports(ch.cfg, m, n, k, align)) return QM_ERR_CONFIG;
-        if (ch.ksplit > 1 && g_configs[ch.cfg].kind != KIND_TILE16) return QM_ERR_CONFIG;
-        ch.ksplit = effective_ksplit(g_configs[ch.cfg], k, ch.ksplit);
-        // partial sums cannot meet in a rounded output: a K split needs the workspace
-        if (ch.ksplit > 1 && !workspace_fits(g_configs[ch.cfg], m, n, ch.ksplit, workspace, workspace_bytes)) return QM_ERR_CONFIG;
-    }
-    if (ch.ksplit > 1) {
-        const hipError_t e = launch_split_with_workspace(p, ch, workspace, s);
-        return e == hipSuccess ? QM_OK : fail_launch(e);
-    }
-    if (cfg == QM_CFG_AUTO && has_ws) {
-        PadPlan pl = plan_padded_k(m, n, k, align, ch);
-        if (pl.on && !scaled_launcher(pl.ch.cfg)) {
-            // a pipelined configuration that has the scaled output, if the shape is one for those
-            const int id = find_config(g_configs[pl.ch.cfg].kind == KIND_TILE16 ? "q256x256_w2x2_s4o1" : "q128x128_w2x2_s4o1");
-            if (id >= 0) pl.ch.cfg = id; else pl.on = false;
-        }
-        if (pl.on && ((uintptr_t)workspace & 15) == 0 && workspace_bytes >= pl.bytes()) {
-            hipError_t e = launch_padded(p, pl, workspace, s);
-            if (e == hipSuccess) e = scaled_launcher(pl.ch.cfg)(p, s, pl.ch.group_m | (1 << 8) | (pl.ch.spread << 16));
-            return e == hipSuccess ? QM_OK : fail_launch(e);
-        }
-    }
-    const LaunchFn launch = scaled_launcher(ch.cfg);
-    if (!launch) return QM_ERR_CONFIG;
-    const hipError_t e = launch(p, s, ch.group_m | (1 << 8) | (ch.spread << 16));
-    return e == hipSuccess ? QM_OK : fail_launch(e);
+    return run_gemm(A, B, D, m, n, k, row_scale, col_scale, out_dtype == QM_OUT_F16 ? OUT_F16 : OUT_BF16,
+                    reinterpret_cast<hipStream_t>(stream), cfg, workspace, workspace_bytes);
 }
 
 QM_EXPORT int qm_gemm_i4_scaled_cfg(const void *A, const void *B, void *D, int m, int n, int k, const float *row_scale,
