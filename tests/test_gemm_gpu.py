@@ -572,3 +572,48 @@ def test_operands_of_two_gib_and_more(oracle_mod):
         assert torch.equal(c_d[:, c0:c0 + cols], part)
     ref = oracle_mod.gemm_i4(a_d.cpu().numpy(), b_d[n - 50:].cpu().numpy())
     assert oracle_mod.compare(np.ascontiguousarray(c_d[:, n - 50:].cpu().numpy()), ref) == -1
+
+
+def test_host_threads_on_their_own_streams():
+    """Four host threads, each with its own stream, operands, output and workspace, call the
+    library at the same time (ctypes drops the GIL for the call): shapes for the pipelined
+    kernel, a K split through the workspace, the skinny and the dot kernel.  Every result of
+    every round equals the one computed alone beforehand."""
+    import threading
+
+    shapes = [(512, 768, 2048), (256, 256, 65536), (16, 4096, 4096), (1, 2048, 8192)]
+    jobs = []
+    for i, (m, n, k) in enumerate(shapes):
+        g = torch.Generator(device=DEV).manual_seed(SEED_BASE + 6300 + i)
+        a_d = torch.randint(-128, 128, (m, k // 2), dtype=torch.int8, device=DEV, generator=g)
+        b_d = torch.randint(-128, 128, (n, k // 2), dtype=torch.int8, device=DEV, generator=g)
+        want = torch.empty((m, n), dtype=torch.int32, device=DEV)
+        qm.gemm(a_d, b_d, want, m, n, k)
+        ws = torch.empty(max(qm.workspace_bytes(m, n, k), 16), dtype=torch.uint8, device=DEV)
+        jobs.append((m, n, k, a_d, b_d, want, ws))
+    torch.cuda.synchronize()
+    assert qm.workspace_bytes(*shapes[1]) > 0
+    failures = []
+
+    def worker(job):
+        m, n, k, a_d, b_d, want, ws = job
+        stream = torch.cuda.Stream(device=DEV)
+        try:
+            with torch.cuda.stream(stream):
+                for _ in range(40):
+                    c_d = poisoned_c(m, n, DEV)
+                    qm.gemm(a_d, b_d, c_d, m, n, k, workspace=ws)
+                    if not torch.equal(c_d, want):
+                        failures.append((m, n, k))
+                        return
+            stream.synchronize()
+        except Exception as ex:  # a thread's exception would otherwise be lost
+            failures.append((m, n, k, repr(ex)))
+
+    threads = [threading.Thread(target=worker, args=(job,)) for job in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert failures == []
