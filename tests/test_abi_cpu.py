@@ -178,3 +178,19 @@ def test_cpu_pack_unpack_mirror_reference_semantics():
     assert torch.equal(qm.unpack_int4(p), v)
     with pytest.raises(qm.QuadmulError):
         qm.pack_int4(torch.zeros(2, 3, dtype=torch.int8))
+
+
+def test_w4a4_linear_argument_checks():
+    """Constructor checks of the linear-layer caller (no GPU: nothing is launched)."""
+    import torch
+    from quadmul_amd.linear import W4A4Linear
+
+    wq = torch.zeros((8, 16), dtype=torch.int8)
+    ws = torch.ones(8, dtype=torch.float32)
+    layer = W4A4Linear(wq, ws, torch.zeros(8), torch.bfloat16)
+    assert (layer.in_features, layer.out_features) == (32, 8) and layer.bias.dtype == torch.bfloat16
+    assert set(layer.state_dict()) == {"weight_packed", "weight_scale", "bias"}
+    for bad in (lambda: W4A4Linear(wq.float(), ws), lambda: W4A4Linear(wq, ws[:4]), lambda: W4A4Linear(wq, ws.double()),
+                lambda: W4A4Linear(wq, ws, torch.zeros(7)), lambda: W4A4Linear(wq, ws, None, torch.float32)):
+        with pytest.raises(qm.QuadmulError):
+            bad()

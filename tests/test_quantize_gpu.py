@@ -71,3 +71,33 @@ def test_int4_linear_layer_end_to_end(oracle_mod):
     ref = x.float() @ w.float().t()
     err = (y.float().cpu() - ref).norm() / ref.norm()
     assert err < 0.25, err  # int4 x int4 with per-row scales: about 15 % relative error on gaussian data
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_w4a4_linear_module(oracle_mod, out_dtype):
+    """The module form of the same chain: leading dimensions flattened, weights quantised once,
+    bias added to the rounded output; bit-exact against the oracle's chain; no rows -> no launch."""
+    from quadmul_amd.linear import W4A4Linear
+
+    n, k = 272, 1056
+    g = torch.Generator().manual_seed(SEED_BASE + 8300)
+    x = (torch.randn((3, 5, k), generator=g) * 0.7).to(torch.bfloat16)
+    w = (torch.randn((n, k), generator=g) * 0.03).to(torch.float32)
+    bias = torch.randn((n,), generator=g).to(out_dtype)
+    layer = W4A4Linear.from_float(w.to(DEV), bias.to(DEV), out_dtype)
+    assert (layer.in_features, layer.out_features) == (k, n) and "bias=True" in repr(layer)
+    y = layer(x.to(DEV))
+    torch.cuda.synchronize()
+    assert y.shape == (3, 5, n) and y.dtype == out_dtype
+    oxq, oxs = oracle_mod.quantize_pack(x.reshape(-1, k).float().numpy())
+    owq, ows = oracle_mod.quantize_pack(w.numpy())
+    out = oracle_mod.OUT_F16 if out_dtype == torch.float16 else oracle_mod.OUT_BF16
+    d = oracle_mod.scale_round16(oracle_mod.gemm_i4(oxq, owq), oxs, ows, out)
+    want = torch.from_numpy(d.view(np.int16)).view(out_dtype) + bias   # one rounded add in the output type
+    assert torch.equal(y.reshape(-1, n).cpu().view(torch.int16), want.view(torch.int16))
+    # the state dict round-trips through the constructor's arguments
+    again = W4A4Linear(layer.weight_packed, layer.weight_scale, layer.bias, out_dtype)
+    assert torch.equal(again(x.to(DEV)), y)
+    assert layer(torch.empty((0, k), dtype=torch.float16, device=DEV)).shape == (0, n)
+    with pytest.raises(qm.QuadmulError):
+        layer(torch.zeros((2, k + 2), dtype=torch.float16, device=DEV))
