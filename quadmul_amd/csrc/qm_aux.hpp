@@ -88,13 +88,31 @@ __global__ void pad_rows_vec_kernel(const v4i *__restrict__ src, v4i *__restrict
     }
 }
 
-__global__ void pad_rows_byte_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, int rows, int kb, int kbp)
+// Source rows at any byte alignment (K / 2 not a multiple of 16, or an operand at an odd
+// address): one wave per row, one 32-bit word of the copy per lane and turn, put together
+// from the two aligned source words that hold its bytes (consecutive lanes read consecutive
+// words), the bytes past the end of the row zeroed.  An aligned word that holds at least one
+// byte of the matrix lies in the same page as that byte, so reading it whole is safe; a word
+// wholly past the end of the matrix is not read.
+__global__ void __launch_bounds__(256) pad_rows_shift_kernel(const uint8_t *__restrict__ src, uint32_t *__restrict__ dst, int rows, int kb, int kbp4)
 {
-    const size_t total = (size_t)rows * kbp;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const size_t r = i / kbp;
-        const int c = (int)(i - r * kbp);
-        dst[i] = c < kb ? src[r * kb + c] : (uint8_t)0;
+    const uintptr_t end = (uintptr_t)src + (size_t)rows * kb;
+    const int lane = threadIdx.x & 63;
+    for (int r = blockIdx.x * 4 + (threadIdx.x >> 6); r < rows; r += gridDim.x * 4) {
+        const uintptr_t at = (uintptr_t)src + (size_t)r * kb;
+        const uint32_t *w = reinterpret_cast<const uint32_t *>(at & ~(uintptr_t)3);
+        const uint32_t shift = (uint32_t)(at & 3);
+        uint32_t *out = dst + (size_t)r * kbp4;
+        for (int q = lane; q < kbp4; q += 64) {
+            const int keep = kb - 4 * q;  // bytes of the row from this word on
+            uint32_t v = 0;
+            if (keep > 0) {
+                const uint32_t x0 = w[q];
+                const uint32_t x1 = (uintptr_t)(w + q + 1) < end ? w[q + 1] : 0u;
+                v = __builtin_amdgcn_alignbyte(x1, x0, shift) & (keep >= 4 ? 0xffffffffu : (1u << (8 * keep)) - 1u);
+            }
+            out[q] = v;
+        }
     }
 }
 

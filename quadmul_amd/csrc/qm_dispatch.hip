@@ -130,8 +130,8 @@ static hipError_t launch_pad_rows(const void *src, void *dst, int rows, int k, i
         const size_t total = (size_t)rows * (kbp / 16);
         pad_rows_vec_kernel<<<dim3(flat_grid(total, 256)), dim3(256), 0, s>>>(static_cast<const v4i *>(src), static_cast<v4i *>(dst), rows, kb / 16, kbp / 16);
     } else {
-        const size_t total = (size_t)rows * kbp;
-        pad_rows_byte_kernel<<<dim3(flat_grid(total, 256)), dim3(256), 0, s>>>(static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), rows, kb, kbp);
+        const unsigned blocks = (unsigned)std::min((rows + 3) / 4, 256 * 32);
+        pad_rows_shift_kernel<<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const uint8_t *>(src), static_cast<uint32_t *>(dst), rows, kb, kbp / 4);
     }
     return hipGetLastError();
 }

@@ -454,7 +454,7 @@ def test_dot_product_kernel_one_and_two_rows(oracle_mod, shape):
     assert oracle_mod.compare(run_gemm(ap, bp, m, n, k), want) == -1
 
 
-@pytest.mark.parametrize("shape", [(3000, 3000, 1056), (1000, 1000, 1000), (300, 5000, 4098), (2100, 4200, 96 + 2)],
+@pytest.mark.parametrize("shape", [(3000, 3000, 1056), (1000, 1000, 1000), (1000, 1100, 1004), (300, 5000, 4098), (2100, 4200, 96 + 2)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_k_padded_through_the_workspace(shape):
     """Large shapes whose K is not a multiple of 32, and unaligned operands: with a workspace
