@@ -73,45 +73,45 @@ __global__ void fill_zero_kernel(int32_t *dst, size_t n)
 }
 
 // --------------------------------------------------------------------------
-// Operand copy with every row padded with zeros to a whole number of 128-nibble K-steps
+// Operand copies with every row padded with zeros to a whole number of 128-nibble K-steps
 // (zero nibbles add nothing to a product): what lets the pipelined kernel run shapes whose
-// K is not a multiple of 128, or whose operands are not 16-byte aligned, out of a
-// caller-provided workspace.  kb / kbp: bytes per row of the source / of the copy.
+// K is not a multiple of 32, or whose operands are not 16-byte aligned, out of a
+// caller-provided workspace.  Both operands in one launch (a second dependent launch costs
+// more than the copy of a small operand): rows 0 .. rows_a-1 are A's, the rest B's.
+// Source rows may start at any byte: one wave per row, one 32-bit word of the copy per
+// lane and turn, put together from the two aligned source words that hold its bytes
+// (consecutive lanes read consecutive words), the bytes past the end of the row zeroed.  An
+// aligned word that holds at least one byte of a matrix lies in the same page as that byte,
+// so reading it whole is safe; a word wholly past the end of the matrix is not read.
+// kb: bytes per source row; kbp4: 32-bit words per row of the copy.
 // --------------------------------------------------------------------------
-__global__ void pad_rows_vec_kernel(const v4i *__restrict__ src, v4i *__restrict__ dst, int rows, int kb16, int kbp16)
-{
-    const size_t total = (size_t)rows * kbp16;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const size_t r = i / kbp16;
-        const int c = (int)(i - r * kbp16);
-        dst[i] = c < kb16 ? src[r * kb16 + c] : v4i{0, 0, 0, 0};
-    }
-}
+struct PadRowsArgs {
+    const uint8_t *src_a, *src_b;
+    uint32_t *dst_a, *dst_b;
+    int rows_a, rows_b, kb, kbp4;
+};
 
-// Source rows at any byte alignment (K / 2 not a multiple of 16, or an operand at an odd
-// address): one wave per row, one 32-bit word of the copy per lane and turn, put together
-// from the two aligned source words that hold its bytes (consecutive lanes read consecutive
-// words), the bytes past the end of the row zeroed.  An aligned word that holds at least one
-// byte of the matrix lies in the same page as that byte, so reading it whole is safe; a word
-// wholly past the end of the matrix is not read.
-__global__ void __launch_bounds__(256) pad_rows_shift_kernel(const uint8_t *__restrict__ src, uint32_t *__restrict__ dst, int rows, int kb, int kbp4)
+__global__ void __launch_bounds__(256) pad_rows_kernel(const PadRowsArgs q)
 {
-    const uintptr_t end = (uintptr_t)src + (size_t)rows * kb;
     const int lane = threadIdx.x & 63;
-    for (int r = blockIdx.x * 4 + (threadIdx.x >> 6); r < rows; r += gridDim.x * 4) {
-        const uintptr_t at = (uintptr_t)src + (size_t)r * kb;
+    for (int r = blockIdx.x * 4 + (threadIdx.x >> 6); r < q.rows_a + q.rows_b; r += gridDim.x * 4) {
+        const bool is_a = r < q.rows_a;
+        const uint8_t *src = is_a ? q.src_a : q.src_b;
+        const int row = is_a ? r : r - q.rows_a;
+        const uintptr_t end = (uintptr_t)src + (size_t)(is_a ? q.rows_a : q.rows_b) * q.kb;
+        const uintptr_t at = (uintptr_t)src + (size_t)row * q.kb;
         const uint32_t *w = reinterpret_cast<const uint32_t *>(at & ~(uintptr_t)3);
         const uint32_t shift = (uint32_t)(at & 3);
-        uint32_t *out = dst + (size_t)r * kbp4;
-        for (int q = lane; q < kbp4; q += 64) {
-            const int keep = kb - 4 * q;  // bytes of the row from this word on
+        uint32_t *out = (is_a ? q.dst_a : q.dst_b) + (size_t)row * q.kbp4;
+        for (int i = lane; i < q.kbp4; i += 64) {
+            const int keep = q.kb - 4 * i;  // bytes of the row from this word on
             uint32_t v = 0;
             if (keep > 0) {
-                const uint32_t x0 = w[q];
-                const uint32_t x1 = (uintptr_t)(w + q + 1) < end ? w[q + 1] : 0u;
+                const uint32_t x0 = w[i];
+                const uint32_t x1 = (uintptr_t)(w + i + 1) < end ? w[i + 1] : 0u;
                 v = __builtin_amdgcn_alignbyte(x1, x0, shift) & (keep >= 4 ? 0xffffffffu : (1u << (8 * keep)) - 1u);
             }
-            out[q] = v;
+            out[i] = v;
         }
     }
 }

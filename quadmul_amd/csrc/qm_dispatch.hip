@@ -123,26 +123,14 @@ static PadPlan plan_padded_k(int m, int n, int k, int ptr_align, const Choice &d
     return pl;
 }
 
-static hipError_t launch_pad_rows(const void *src, void *dst, int rows, int k, int kp, hipStream_t s)
-{
-    const int kb = k / 2, kbp = kp / 2;
-    if (kb % 16 == 0 && ((uintptr_t)src & 15) == 0) {
-        const size_t total = (size_t)rows * (kbp / 16);
-        pad_rows_vec_kernel<<<dim3(flat_grid(total, 256)), dim3(256), 0, s>>>(static_cast<const v4i *>(src), static_cast<v4i *>(dst), rows, kb / 16, kbp / 16);
-    } else {
-        const unsigned blocks = (unsigned)std::min((rows + 3) / 4, 256 * 32);
-        pad_rows_shift_kernel<<<dim3(blocks), dim3(256), 0, s>>>(static_cast<const uint8_t *>(src), static_cast<uint32_t *>(dst), rows, kb, kbp / 4);
-    }
-    return hipGetLastError();
-}
-
 // The padded copies of A and B in the workspace, and the arguments of the GEMM on them.
 static hipError_t launch_padded(GemmArgs &p, const PadPlan &pl, void *ws, hipStream_t s)
 {
     uint8_t *a_p = static_cast<uint8_t *>(ws), *b_p = a_p + pl.a_bytes;
-    hipError_t e = launch_pad_rows(p.A, a_p, p.M, p.K, pl.kp, s);
-    if (e != hipSuccess) return e;
-    e = launch_pad_rows(p.B, b_p, p.N, p.K, pl.kp, s);
+    const PadRowsArgs q{p.A, p.B, reinterpret_cast<uint32_t *>(a_p), reinterpret_cast<uint32_t *>(b_p), p.M, p.N, p.K / 2, pl.kp / 8};
+    const long long rows = (long long)p.M + p.N;
+    pad_rows_kernel<<<dim3((unsigned)std::min<long long>((rows + 3) / 4, 256 * 32)), dim3(256), 0, s>>>(q);
+    const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     p.A = a_p;
     p.B = b_p;
