@@ -24,6 +24,16 @@ template <class Cfg>
 static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
 {
     const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
+    // More column blocks than two workgroups per CU can hold at once, and K within one turn
+    // of the waves: workgroups that walk over several blocks each, evenly.
+    constexpr int resident = 2 * 256;
+    if constexpr (Cfg::U % 2 == 0) {
+        if (blocks > resident && (p.K + 127) / 128 <= Cfg::NW * Cfg::U) {
+            const int turns = (blocks + resident - 1) / resident;
+            gemm_skinny_stream_kernel<Cfg><<<dim3((blocks + turns - 1) / turns), dim3(Cfg::THREADS), 0, stream>>>(p, blocks);
+            return hipGetLastError();
+        }
+    }
     gemm_skinny_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), 0, stream>>>(p);
     return hipGetLastError();
 }

@@ -617,3 +617,34 @@ def test_host_threads_on_their_own_streams():
         t.join()
     torch.cuda.synchronize()
     assert failures == []
+
+
+@pytest.mark.parametrize("shape", [(16, 11008, 4096), (3, 8210, 1024), (128, 8195, 1056), (40, 16400, 2048), (1, 24577, 512)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_skinny_kernel_walking_over_column_blocks(oracle_mod, shape):
+    """More column blocks than two workgroups per CU hold at once and K within one turn of the
+    waves: the skinny kernel's workgroups walk over several blocks each, A fragments kept,
+    B of the next block prefetched, sums in alternating halves of the LDS.  Every skinny
+    configuration that takes the shape, int32 and scaled output, against the oracle."""
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 6500 + n)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    g = torch.Generator().manual_seed(SEED_BASE + 6600 + n)
+    rs, cs = torch.rand(m, generator=g) * 0.01 + 0.001, torch.rand(n, generator=g) + 0.5
+    want16 = oracle_mod.scale_round16(want, rs.numpy(), cs.numpy(), oracle_mod.OUT_BF16)
+    ran = 0
+    for cfg, name in enumerate(qm.config_names()):
+        if not name.startswith("s") or not qm.config_supports(cfg, m, n, k):
+            continue
+        c_d = poisoned_c(m, n, DEV)
+        qm.gemm_cfg(a_d, b_d, c_d, m, n, k, cfg)
+        d_d = torch.zeros((m, n), dtype=torch.bfloat16, device=DEV)
+        qm.gemm_scaled(a_d, b_d, d_d, m, n, k, rs.to(DEV), cs.to(DEV), cfg)
+        torch.cuda.synchronize()
+        bad = oracle_mod.compare(c_d.cpu().numpy(), want)
+        assert bad == -1, f"{name}: first mismatch at flat index {bad}"
+        assert np.array_equal(d_d.view(torch.int16).cpu().numpy().view(np.uint16), want16), name
+        ran += 1
+    assert ran >= 2
