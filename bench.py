@@ -106,8 +106,8 @@ def time_graph(fn, launches=200, replays=5):
 # Bytes moved per launch past the L2s, from rocprofv3 counter runs of `bench.py --workload W
 # --launches-only 20` (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads
 # for a 256 MiB device-to-device copy; summaries under profiles/).  Not measured live.
-MEASURED_TRAFFIC = {(4096, 4096, 4096): 118965218, (8192, 8192, 8192): 677409906, (16, 4096, 4096): 8952208, (1, 4096, 4096): 8455592}
-MEASURED_TRAFFIC_OTHER = {"scaled_fp16_4096^3": 84838220, "quantize_pack_fp16_4096x4096": 42116169}
+MEASURED_TRAFFIC = {(4096, 4096, 4096): 118964029, (8192, 8192, 8192): 677540868, (16, 4096, 4096): 8956310, (1, 4096, 4096): 8455598}
+MEASURED_TRAFFIC_OTHER = {"scaled_fp16_4096^3": 84835801, "quantize_pack_fp16_4096x4096": 42113123}
 
 
 def roofline_of(m, n, k, bound, ms):
