@@ -271,21 +271,24 @@ gemm_skinny_stream_kernel(const GemmArgs p, const int nblocks)
 #pragma unroll
             for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            v4i bev[FN], bod[FN];
+        for (int pu = 0; pu < PAIRS; ++pu) {
+            v4i bev[2][FN], bod[2][FN];
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
                 v4i q0, q1;
-                chunks_from_halves(bl[u / 2][j][0], bl[u / 2][j][1], q0, q1);
-                x16_expand(lane_gather(u % 2 ? q1 : q0, u % 2 ? from_c1 : from_c0), bev[j], bod[j]);
+                chunks_from_halves(bl[pu][j][0], bl[pu][j][1], q0, q1);
+                x16_expand(lane_gather(q0, from_c0), bev[0][j], bod[0][j]);
+                x16_expand(lane_gather(q1, from_c1), bev[1][j], bod[1][j]);
             }
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
+            for (int c = 0; c < 2; ++c)
 #pragma unroll
-                for (int j = 0; j < FN; ++j) acc[i][j] = mfma16(bev[j], aev[u][i], acc[i][j]);
+                for (int i = 0; i < FM; ++i) {
 #pragma unroll
-                for (int j = 0; j < FN; ++j) acc[i][j] = mfma16(bod[j], aod[u][i], acc[i][j]);
-            }
+                    for (int j = 0; j < FN; ++j) acc[i][j] = mfma16(bev[c][j], aev[2 * pu + c][i], acc[i][j]);
+#pragma unroll
+                    for (int j = 0; j < FN; ++j) acc[i][j] = mfma16(bod[c][j], aod[2 * pu + c][i], acc[i][j]);
+                }
         }
 #pragma unroll
         for (int i = 0; i < FM; ++i)
