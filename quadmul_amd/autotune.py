@@ -96,10 +96,18 @@ def random_packed(rows: int, k: int, seed: int, device) -> torch.Tensor:
 
 
 def tune_shape(m: int, n: int, k: int, device, group_ms: Iterable[int], min_ms: float, reps: int, verbose: bool,
-               only: str = "") -> Dict:
+               only: str = "", rotate_mib: int = 0) -> Dict:
+    """Time every configuration that takes the shape.  ``rotate_mib`` > 0: the timed launches
+    rotate over as many copies of B (each with its own C) as fill that many MiB, so that B
+    comes from HBM and not from the L2s and the 256 MiB memory-side cache -- what a weight
+    matrix does in a model of many layers; 0 times all launches on one B, as the reference's
+    harness does (test.py:78-91)."""
     a = random_packed(m, k, 1, device)
     b = random_packed(n, k, 2, device)
     c = torch.empty((m, n), dtype=torch.int32, device=device)
+    ncopies = max(1, -(-(rotate_mib << 20) // max(1, b.numel()))) if rotate_mib > 0 else 1
+    bs = [b] + [b.clone() for _ in range(ncopies - 1)]
+    cs = [c] + [torch.empty_like(c) for _ in range(ncopies - 1)]
     # Cross-check: the generic kernel where it finishes quickly, else the first candidate
     # (parity against the CPU oracle is the test-suite's job, not the tuner's).
     ref = None
@@ -134,7 +142,14 @@ def tune_shape(m: int, n: int, k: int, device, group_ms: Iterable[int], min_ms: 
                 ref = c.clone()
             if not torch.equal(c, ref):
                 raise RuntimeError(f"{name} group_m={gm} ksplit={ks} spread={spread} disagrees with the cross-check result on {m}x{n}x{k}")
-            ms = time_launches(lambda: qm.gemm_cfg(a, b, c, m, n, k, code), min_ms, reps)
+            turn = [0]
+
+            def launch():
+                i = turn[0] % ncopies
+                turn[0] += 1
+                qm.gemm_cfg(a, bs[i], cs[i], m, n, k, code)
+
+            ms = time_launches(launch, min_ms, reps)
             results.append({"config": name, "group_m": gm, "ksplit": ks, "spread": spread, "ms": ms, "tops": ops / ms / 1e9,
                             "gbs": algorithmic_bytes(m, n, k) / ms / 1e6})
             if verbose:
@@ -184,6 +199,8 @@ def main(argv=None) -> int:
     ap.add_argument("--json", default=None, help="write all measurements here")
     ap.add_argument("--emit", default=None, help="write the table rows here (csrc/qm_tile_table.inc format)")
     ap.add_argument("--only", default="", help="regular expression: time only configurations whose name matches")
+    ap.add_argument("--rotate-b", type=int, default=0, metavar="MiB",
+                    help="rotate the timed launches over copies of B filling this many MiB (e.g. 320: B then comes from HBM)")
     ap.add_argument("-v", "--verbose", action="store_true")
     a = ap.parse_args(argv)
     if not torch.cuda.is_available():
@@ -192,7 +209,7 @@ def main(argv=None) -> int:
     device = torch.device("cuda:0")
     gms = [int(x) for x in a.group_m.split(",")]
     t0 = time.time()
-    tuned = [tune_shape(m, n, k, device, gms, a.min_ms, a.reps, a.verbose, a.only) for (m, n, k) in parse_shapes(a.shapes)]
+    tuned = [tune_shape(m, n, k, device, gms, a.min_ms, a.reps, a.verbose, a.only, a.rotate_b) for (m, n, k) in parse_shapes(a.shapes)]
     print(f"tuned {len(tuned)} shapes in {time.time()-t0:.0f} s on {torch.cuda.get_device_name(0)}", flush=True)
     if a.json:
         with open(a.json, "w") as f:
