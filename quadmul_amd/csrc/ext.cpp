@@ -169,22 +169,33 @@ void gemm_scaled_op(const torch::Tensor &a, const torch::Tensor &b, torch::Tenso
     gemm_scaled(a, b, d, m, n, k, row_scale, col_scale);
 }
 
+// quantize_pack returns new tensors: the Meta form only has to give their shapes and types
+std::tuple<torch::Tensor, torch::Tensor> quantize_pack_meta(const torch::Tensor &x)
+{
+    TORCH_CHECK(x.dim() == 2 && x.size(1) % 2 == 0, "quadmul.quantize_pack: expects a 2-D tensor with even K");
+    return {torch::empty({x.size(0), x.size(1) / 2}, x.options().dtype(torch::kInt8)), torch::empty({x.size(0)}, x.options().dtype(torch::kFloat32))};
+}
+std::tuple<torch::Tensor, torch::Tensor> quantize_pack_op(const torch::Tensor &x) { return quantize_pack(x); }
+
 }  // namespace
 
 TORCH_LIBRARY(quadmul, m)
 {
     m.def("gemm(Tensor a, Tensor b, Tensor(c!) c, int m, int n, int k) -> ()");
     m.def("gemm_scaled(Tensor a, Tensor b, Tensor(d!) d, int m, int n, int k, Tensor? row_scale, Tensor? col_scale) -> ()");
+    m.def("quantize_pack(Tensor x) -> (Tensor, Tensor)");
 }
 TORCH_LIBRARY_IMPL(quadmul, CUDA, m)
 {
     m.impl("gemm", &gemm_op);
     m.impl("gemm_scaled", &gemm_scaled_op);
+    m.impl("quantize_pack", &quantize_pack_op);
 }
 TORCH_LIBRARY_IMPL(quadmul, Meta, m)
 {
     m.impl("gemm", &gemm_meta);
     m.impl("gemm_scaled", &gemm_scaled_meta);
+    m.impl("quantize_pack", &quantize_pack_meta);
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)

@@ -101,3 +101,29 @@ def test_w4a4_linear_module(oracle_mod, out_dtype):
     assert layer(torch.empty((0, k), dtype=torch.float16, device=DEV)).shape == (0, n)
     with pytest.raises(qm.QuadmulError):
         layer(torch.zeros((2, k + 2), dtype=torch.float16, device=DEV))
+
+
+def test_linear_chain_through_dispatcher_ops_traced(oracle_mod):
+    """quantize_pack and gemm_scaled as dispatcher ops: the whole linear chain stays in one
+    traced graph (aot_eager: fake tensors go through the Meta implementations) and gives the
+    oracle's bits."""
+    import quadmul  # noqa: F401
+
+    m, n, k = 48, 96, 512
+    g = torch.Generator().manual_seed(SEED_BASE + 8400)
+    x = (torch.randn((m, k), generator=g) * 0.5).to(torch.float16)
+    w = (torch.randn((n, k), generator=g) * 0.05).to(torch.float16)
+    wq, ws = torch.ops.quadmul.quantize_pack(w.to(DEV))
+
+    def fn(x_, wq_, ws_):
+        xq, xs = torch.ops.quadmul.quantize_pack(x_)
+        y = torch.empty((m, n), dtype=torch.float16, device=x_.device)
+        torch.ops.quadmul.gemm_scaled(xq, wq_, y, m, n, k, xs, ws_)
+        return y
+
+    y = torch.compile(fn, backend="aot_eager", fullgraph=True)(x.to(DEV), wq, ws)
+    torch.cuda.synchronize()
+    oxq, oxs = oracle_mod.quantize_pack(x.float().numpy())
+    owq, ows = oracle_mod.quantize_pack(w.float().numpy())
+    want = oracle_mod.scale_round16(oracle_mod.gemm_i4(oxq, owq), oxs, ows, oracle_mod.OUT_F16)
+    assert (y.view(torch.int16).cpu().numpy().view(np.uint16) == want).all()
