@@ -35,6 +35,8 @@ WORKLOADS = {
     "square8192": (8, 8192, 8192, 8192, "mfma"),
     "skinny16": (3, 16, 4096, 4096, "hbm"),
     "skinny1": (2, 1, 4096, 4096, "hbm"),
+    # the skinny target's kernel at a size where the launch no longer dominates (an extra, not a BASELINE row)
+    "skinny16_wide": (4, 16, 28672, 4096, "hbm"),
 }
 
 
