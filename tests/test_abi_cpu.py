@@ -145,6 +145,11 @@ def test_selection_rules():
     for m in (16, 64):
         assert name(m, 4096, 4096).startswith("s"), m
     assert name(1, 4096, 4096).startswith("v") and name(2, 5120, 5120).startswith("v")   # dot-product kernel
+    # up to 32 rows: the skinny kernel whatever N and K; 33..64 rows: four row blocks while the
+    # 64-row tiles number one per CU at most, beyond that whichever the cost model prices lower
+    assert name(9, 28672, 14336) == "s1x1_w16_u2" and name(32, 11008, 4096) == "s2x1_w8_u4" and name(24, 4096, 8192) == "s2x1_w16_u2"
+    assert name(40, 11008, 14336) == "s4x1_w8_u2" and name(64, 14336, 4096) == "s4x1_w16_u2" and name(64, 4096, 4096) == "s4x1_w16_u1"
+    assert name(64, 28672, 14336).startswith("q")
     # few tiles, long K: the pipelined kernel with K split over several workgroups per tile
     code = qm.select_config(128, 8192, 28672)
     assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
