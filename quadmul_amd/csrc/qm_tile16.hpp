@@ -125,7 +125,7 @@ struct Tile16Cfg {
     static constexpr int PITCH = 64;                  // packed bytes per row per K-step
     static constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-    static constexpr int STAGES = STAGES_;  // LDS ring depth: 4, or 5 for one more K-step of DMA latency cover
+    static constexpr int STAGES = STAGES_;  // LDS ring depth: 4 or 5 on the large tiles; 6 to 8 on the small ones, whose K-steps are short against the latency of HBM
     static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
     // Per-wave LDS area through which finished accumulator blocks are turned into row-major
     // order before they are stored: 16 rows x 64 int32, rows padded by 16 bytes so that the
@@ -139,7 +139,7 @@ struct Tile16Cfg {
     static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile is a multiple of 16x16");
     static_assert(BM % (16 * WAVES) == 0 && BN % (16 * WAVES) == 0, "DMA pieces must divide evenly among the waves");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
-    static_assert(STAGES >= 3 && STAGES <= 5, "ring depth");
+    static_assert(STAGES >= 3 && STAGES <= 8, "ring depth");
     static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
     static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
     static_assert((W_OPS * FN) % FM == 0, "B widening must split evenly over the sub-steps");

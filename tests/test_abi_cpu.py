@@ -69,7 +69,7 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4(None, None, None, 0, 4, 4, None) == 0    # empty: nothing to do
     assert lib.qm_gemm_i4(None, None, None, 4, 0, 4, None) == 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 4, 4, 4, None, 9999) == -3
-    assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("q128x128_w2x2_s4o1")) == -3   # K % 32 != 0
+    assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("q128x128_w2x2_s7o1")) == -3   # K % 32 != 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 96, None, qm.config_id("q256x256_w2x2_s4o1")) == -3   # a single short K-step
     assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
     assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
@@ -103,7 +103,7 @@ def test_status_codes_without_a_gpu():
 
 
 def test_workspace_sizes():
-    q128 = qm.config_id("q128x128_w2x2_s4o1")
+    q128 = qm.config_id("q128x128_w2x2_s7o1")
     # one padded int32 tile per (split, tile): 2 x 3 tiles of 128 x 128, 4 splits
     assert qm.workspace_bytes(200, 300, 4096, q128 | (4 << 24)) == 4 * 6 * 128 * 128 * 4
     # splits without work do not count: 3 K-steps cannot feed 8 splits

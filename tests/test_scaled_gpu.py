@@ -90,9 +90,9 @@ def test_rejections():
     with pytest.raises(qm.QuadmulError):  # the 256 x 128 tile two to a CU has no scaled output (its registers do not hold the scales)
         qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q256x128_w2x2_s3o2"))
     with pytest.raises(qm.QuadmulError):  # partial sums cannot meet in a rounded output: a K split needs a workspace
-        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s4o1") | (2 << 24), workspace=None)
+        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s7o1") | (2 << 24), workspace=None)
     with pytest.raises(qm.QuadmulError):
-        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s4o1") | (2 << 24),
+        qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("q128x128_w2x2_s7o1") | (2 << 24),
                        workspace=torch.empty(1024, dtype=torch.uint8, device=DEV))
     with pytest.raises(qm.QuadmulError):  # only the pipelined kernel splits K
         qm.gemm_scaled(a, a, d, m, n, k, None, None, names.index("s4x1_w8_u2") | (2 << 24))
