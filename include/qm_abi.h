@@ -38,6 +38,8 @@ extern "C" {
 #define QM_ERR_LAUNCH        -4 /* the HIP runtime refused the launch (see qm_last_hip_error) */
 #define QM_ERR_ALIGN         -5 /* C is not 4-byte aligned (a 16-bit output: 2-byte)         */
 #define QM_ERR_DTYPE         -6 /* out_dtype is none of the QM_OUT_* values                 */
+#define QM_ERR_SCRATCH       -7 /* qm_gemm_i4_static: the call needs more scratch memory than
+                                   QM_STATIC_SCRATCH_BYTES                                   */
 
 #define QM_CFG_AUTO          -1 /* let the shape table / heuristic choose                   */
 
@@ -118,6 +120,29 @@ int qm_gemm_i4_scaled_ws(const void *A, const void *B, void *D, int m, int n, in
                          const float *col_scale, int out_dtype, void *stream, int cfg, void *workspace,
                          size_t workspace_bytes);
 size_t qm_gemm_workspace_bytes(int m, int n, int k, int ptr_align, int cfg, int scaled);
+
+/*
+ * qm_gemm_i4 for callers that cannot allocate and have no workspace to lend: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in
+ * the reference (its wrapper, kernel.cu:334, never needs scratch memory because it never
+ * splits K and skips the shapes it has no table row for).  Runs exactly what
+ * qm_gemm_i4_ws(..., QM_CFG_AUTO, workspace, bytes) runs when it is lent a workspace of
+ * qm_gemm_workspace_bytes(m, n, k, align, QM_CFG_AUTO, 0) bytes -- same kernels, same result
+ * bit for bit -- but the partial tiles of a K split and the zero-padded operand copies live
+ * in an array of QM_STATIC_SCRATCH_BYTES that is part of the library's device code: every
+ * GPU the library runs on holds one copy of it from the first kernel launch until the
+ * process ends.  The call makes no hipMalloc / hipFree and no other allocating call.
+ *   - A call that would use more than QM_STATIC_SCRATCH_BYTES returns QM_ERR_SCRATCH and
+ *     enqueues nothing (use qm_gemm_i4_ws with a workspace of your own, or qm_gemm_i4).
+ *   - All calls on one GPU share that GPU's array: calls on ONE stream are ordered and
+ *     safe; calls that may overlap on the GPU (different streams, no dependency) race on
+ *     it and must not both use this entry point.  Nothing in the array has to start from
+ *     zero (every byte a kernel reads was written by an earlier kernel of the same call).
+ *   - The first call on a device looks the array's address up (hipGetSymbolAddress); make
+ *     one call per device before capturing this entry point into a graph.
+ */
+#define QM_STATIC_SCRATCH_BYTES (64u << 20)
+int qm_gemm_i4_static(const void *A, const void *B, void *C, int m, int n, int k, void *stream);
 
 /* The configuration qm_gemm_i4_ws picks for this shape when it is given a workspace
  * (the table lookup the reference does at kernel.cu:340-385, here with a heuristic

@@ -21,7 +21,7 @@ from typing import List, Optional
 import torch
 
 __all__ = [
-    "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "gemm_scaled", "pack_int4", "unpack_int4",
+    "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "gemm_static", "gemm_scaled", "pack_int4", "unpack_int4",
     "config_has_scaled", "quantize_pack",
     "num_configs", "config_name", "config_names", "config_id", "select_config", "config_supports",
     "CFG_AUTO", "version",
@@ -35,7 +35,7 @@ CFG_AUTO = -1
 #: every symbol include/qm_abi.h declares
 ABI_SYMBOLS = (
     "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled",
-    "qm_gemm_i4_ws", "qm_gemm_i4_scaled_ws", "qm_gemm_workspace_bytes", "qm_quantize_pack_i4", "qm_select_config", "qm_num_configs", "qm_config_name",
+    "qm_gemm_i4_ws", "qm_gemm_i4_static", "qm_gemm_i4_scaled_ws", "qm_gemm_workspace_bytes", "qm_quantize_pack_i4", "qm_select_config", "qm_num_configs", "qm_config_name",
     "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version",
 )
 
@@ -69,6 +69,8 @@ def library() -> ctypes.CDLL:
     lib.qm_gemm_i4_scaled_cfg.restype = ci
     lib.qm_gemm_i4_ws.argtypes = [vp, vp, vp, ci, ci, ci, vp, ci, vp, ctypes.c_size_t]
     lib.qm_gemm_i4_ws.restype = ci
+    lib.qm_gemm_i4_static.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+    lib.qm_gemm_i4_static.restype = ci
     lib.qm_gemm_i4_scaled_ws.argtypes = [vp, vp, vp, ci, ci, ci, vp, vp, ci, vp, ci, vp, ctypes.c_size_t]
     lib.qm_gemm_i4_scaled_ws.restype = ci
     lib.qm_gemm_workspace_bytes.argtypes = [ci, ci, ci, ci, ci, ci]
@@ -238,6 +240,20 @@ def gemm(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: i
     without one (the splits then meet in ``c`` through atomics); a uint8 tensor is used as
     it is.  The result is the same in every case."""
     gemm_cfg(a, b, c, m, n, k, CFG_AUTO, workspace)
+
+
+STATIC_SCRATCH_BYTES = 64 << 20
+
+
+def gemm_static(a: torch.Tensor, b: torch.Tensor, c: torch.Tensor, m: int, n: int, k: int) -> None:
+    """:func:`gemm` through ``qm_gemm_i4_static``: nothing is allocated, the scratch memory of
+    a K split or of zero-padded operand copies is an array inside the library (at most
+    ``STATIC_SCRATCH_BYTES``; beyond that the call raises).  Calls that may overlap on one GPU
+    race on that array: keep them on one stream."""
+    _check_operands(a, b, c, m, n, k)
+    with torch.cuda.device(a.device):
+        st = library().qm_gemm_i4_static(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, n, k, _stream_ptr(a))
+    _check(st, "qm_gemm_i4_static")
 
 
 def pack_int4(values: torch.Tensor) -> torch.Tensor:

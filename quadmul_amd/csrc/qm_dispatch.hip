@@ -296,6 +296,48 @@ QM_EXPORT int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n,
     return run_gemm(A, B, C, m, n, k, nullptr, nullptr, OUT_I32, reinterpret_cast<hipStream_t>(stream), cfg, workspace, workspace_bytes);
 }
 
+// --------------------------------------------------------------------------
+// Library-owned scratch memory for qm_gemm_i4_static.  In host code the array's name is only
+// a handle for hipGetSymbolAddress: every device has its own copy at its own address, looked
+// up once per device (with that device current) and kept; kernels and every other use take
+// that pointer.
+// --------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[QM_STATIC_SCRATCH_BYTES];
+static std::atomic<void *> g_scratch_ptr[QM_MAX_DEVICES] = {};
+
+static hipError_t static_scratch(void **out)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= QM_MAX_DEVICES) return hipErrorInvalidDevice;
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (ptr == nullptr || ((uintptr_t)ptr & 255) != 0) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return hipSuccess;
+}
+
+QM_EXPORT int qm_gemm_i4_static(const void *A, const void *B, void *C, int m, int n, int k, void *stream)
+{
+    const int st = check_gemm_args(A, B, C, m, n, k);
+    if (st != QM_OK) return st;
+    if (m == 0 || n == 0) return QM_OK;
+    const size_t need = qm_gemm_workspace_bytes(m, n, k, ptr_alignment(A, B), QM_CFG_AUTO, 0);
+    if (need > (size_t)QM_STATIC_SCRATCH_BYTES) return QM_ERR_SCRATCH;
+    void *ws = nullptr;
+    if (need > 0) {
+        const hipError_t e = static_scratch(&ws);
+        if (e != hipSuccess) return fail_launch(e);
+    }
+    return run_gemm(A, B, C, m, n, k, nullptr, nullptr, OUT_I32, reinterpret_cast<hipStream_t>(stream), QM_CFG_AUTO, ws,
+                    ws ? (size_t)QM_STATIC_SCRATCH_BYTES : 0);
+}
+
 QM_EXPORT int qm_gemm_i4_cfg(const void *A, const void *B, void *C, int m, int n, int k, void *stream, int cfg)
 {
     return qm_gemm_i4_ws(A, B, C, m, n, k, stream, cfg, nullptr, 0);
@@ -438,6 +480,7 @@ QM_EXPORT const char *qm_status_string(int status)
     case QM_ERR_LAUNCH: return "HIP launch failed";
     case QM_ERR_ALIGN: return "C must be 4-byte aligned (a 16-bit output 2-byte aligned)";
     case QM_ERR_DTYPE: return "unknown output type";
+    case QM_ERR_SCRATCH: return "the call needs more scratch memory than the library's static array (QM_STATIC_SCRATCH_BYTES) holds";
     default: return "unknown status";
     }
 }

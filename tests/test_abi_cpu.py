@@ -71,6 +71,13 @@ def test_status_codes_without_a_gpu():
     assert lib.qm_gemm_i4_cfg(one, one, one, 4, 4, 4, None, 9999) == -3
     assert lib.qm_gemm_i4_cfg(one, one, one, 128, 128, 30, None, qm.config_id("q128x128_w2x2_s7o1")) == -3   # K % 32 != 0
     assert lib.qm_gemm_i4_cfg(one, one, one, 256, 256, 96, None, qm.config_id("q256x256_w2x2_s4o1")) == -3   # a single short K-step
+    # the entry point on the library's own scratch array: same checks, and a call that would
+    # need more than the array holds is refused before anything touches the GPU
+    assert lib.qm_gemm_i4_static(one, one, one, 4, 4, 3, None) == -2
+    assert lib.qm_gemm_i4_static(one, one, None, 4, 4, 4, None) == -1
+    assert lib.qm_gemm_i4_static(None, None, None, 0, 4, 4, None) == 0
+    assert qm.workspace_bytes(16384, 16384, 8100) > qm.STATIC_SCRATCH_BYTES
+    assert lib.qm_gemm_i4_static(one, one, one, 16384, 16384, 8100, None) == -7
     assert lib.qm_pack_i4(one, one, 4, 3, None) == -2
     assert lib.qm_pack_i4(None, None, 0, 8, None) == 0
     assert lib.qm_unpack_i4(None, one, 4, 8, None) == -1
