@@ -28,6 +28,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIBDIR = os.path.join(PKG, "lib")
 OBJDIR = os.path.join(PKG, "build")
 LIB_PATH = os.path.join(LIBDIR, "libqm_hip.so")
+PROBE_PATH = os.path.join(LIBDIR, "libqm_probe.so")
 N_TILE_TUS = 12
 
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
@@ -70,6 +71,16 @@ def build_lib(jobs: int = 8, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+def build_probe(verbose: bool = False) -> str:
+    """The measurement probes of bench.py (MFMA issue rate, launch floor, read floor): a
+    library of their own, not linked into libqm_hip.so."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    out = _run([HIPCC] + HIP_FLAGS + ["-shared", os.path.join(CSRC, "qm_probe.hip"), "-o", PROBE_PATH])
+    if verbose and out.strip():
+        print(out)
+    return PROBE_PATH
+
+
 def build_ext(verbose: bool = False) -> str:
     import torch
     from torch.utils import cpp_extension
@@ -94,7 +105,7 @@ def build_ext(verbose: bool = False) -> str:
 
 
 def build_all(jobs: int = 8, verbose: bool = False):
-    return build_lib(jobs, verbose), build_ext(verbose)
+    return build_lib(jobs, verbose), build_probe(verbose), build_ext(verbose)
 
 
 def main(argv=None):
@@ -106,6 +117,7 @@ def main(argv=None):
     a = ap.parse_args(argv)
     if a.lib or not a.ext:
         print("built", build_lib(a.jobs, a.verbose))
+        print("built", build_probe(a.verbose))
     if a.ext or not a.lib:
         print("built", build_ext(a.verbose))
     return 0

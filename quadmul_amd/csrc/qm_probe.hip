@@ -1,0 +1,105 @@
+// Measurement probes for bench.py (libqm_probe.so): what the part itself sustains, to set
+// beside the nominal peaks the roofline fractions are quoted against.  Not part of the GEMM
+// library and not linked into it.  The timing method follows the reference's own harness
+// (kernel.cu:468-497: warm-ups, then launches between two events), with the kernels below
+// in place of the GEMM.
+//
+//   qm_probe_mfma_issue   a loop of independent v_mfma_i32_16x16x64_i8 on operands of the
+//                         form 16 * s4 (low nibble zero), the instruction and the operand
+//                         form of the GEMM kernels, with nothing else in the loop: the
+//                         issue peak of the matrix cores at the clock the part sustains
+//   qm_probe_empty        a kernel that does nothing: the launch floor
+//   qm_probe_read         a kernel that only reads `bytes` (16 bytes per lane, whole lines)
+//                         and keeps a checksum: the floor of "launch + one pass over B"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define QM_PROBE_EXPORT extern "C" __attribute__((visibility("default")))
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int MFMA_PER_ITER = 16;   // independent accumulators: 16 x 4 AGPRs
+constexpr int MFMA_OPS = 2 * 16 * 16 * 64;
+
+// One workgroup of four waves (one per SIMD) per launch slot; `iters` trips of 16 MFMAs.
+// out[2 * block], out[2 * block + 1]: what the two counters of the core (s_memtime) and of
+// the constant 100 MHz reference (s_memrealtime) advanced by around the loop, from wave 0.
+__global__ void __launch_bounds__(256) mfma_issue_kernel(uint64_t *out, int iters, uint32_t seed)
+{
+    // pseudo-random nibbles in the high half of every byte: the matrix cores draw power by
+    // the bits that toggle, so all-zero operands would flatter the result
+    uint32_t h = (threadIdx.x + 1) * 2654435761u + blockIdx.x * 40503u + seed;
+    v4i s0, s1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        h ^= h << 13; h ^= h >> 17; h ^= h << 5;
+        s0[i] = (int)(h & 0xF0F0F0F0u);
+        h ^= h << 13; h ^= h >> 17; h ^= h << 5;
+        s1[i] = (int)(h & 0xF0F0F0F0u);
+    }
+    v4i acc[MFMA_PER_ITER];
+#pragma unroll
+    for (int i = 0; i < MFMA_PER_ITER; ++i) acc[i] = v4i{0, 0, 0, 0};
+    const uint64_t t0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < MFMA_PER_ITER; ++i)
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(s0), "v"(s1));
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    const uint64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < MFMA_PER_ITER; ++i) sum += acc[i].x ^ acc[i].y ^ acc[i].z ^ acc[i].w;
+    if (threadIdx.x == 0) {
+        out[2 * blockIdx.x] = t1 - t0;
+        out[2 * blockIdx.x + 1] = r1 - r0;
+    }
+    if (sum == 0x7fffffff && iters < 0) out[0] = (uint64_t)sum;  // keeps the accumulators alive
+}
+
+__global__ void empty_kernel() {}
+
+__global__ void __launch_bounds__(256) read_kernel(const v4i *src, size_t n16, int *sink)
+{
+    v4i acc = {0, 0, 0, 0};
+    const size_t stride = (size_t)gridDim.x * 256 * 4;
+    for (size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x; i < n16; i += stride) {
+        v4i v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = i + u * 256 < n16 ? __builtin_nontemporal_load(src + i + u * 256) : v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc ^= v[u];
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5A5A5A5B) *sink = 1;  // (practically never: keeps the loads)
+}
+
+}  // namespace
+
+// Enqueues one launch of `blocks` workgroups x 4 waves x iters x 16 MFMAs.  out: device
+// memory for 2 * blocks uint64.  Returns the integer operations of the launch (2 * 16 * 16
+// * 64 per MFMA per wave) as a double, or a negative hipError_t.
+QM_PROBE_EXPORT double qm_probe_mfma_issue(void *out, int blocks, int iters, void *stream)
+{
+    if (!out || blocks < 1 || iters < 1) return -1.0;
+    mfma_issue_kernel<<<dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(static_cast<uint64_t *>(out), iters, 12345u);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return -(double)(int)e;
+    return (double)blocks * 4.0 * (double)iters * MFMA_PER_ITER * (double)MFMA_OPS;
+}
+
+QM_PROBE_EXPORT int qm_probe_empty(void *stream)
+{
+    empty_kernel<<<dim3(1), dim3(64), 0, reinterpret_cast<hipStream_t>(stream)>>>();
+    return (int)hipGetLastError();
+}
+
+// `src`: 16-byte aligned device memory of `bytes` bytes (a multiple of 16); `sink`: one int.
+QM_PROBE_EXPORT int qm_probe_read(const void *src, size_t bytes, void *sink, int blocks, void *stream)
+{
+    if (!src || !sink || (bytes & 15) || ((uintptr_t)src & 15) || blocks < 1) return -1;
+    read_kernel<<<dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(static_cast<const v4i *>(src), bytes / 16, static_cast<int *>(sink));
+    return (int)hipGetLastError();
+}
