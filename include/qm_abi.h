@@ -149,6 +149,10 @@ int qm_gemm_i4_static(const void *A, const void *B, void *C, int m, int n, int k
  * fallback instead of a silent no-op); without a workspace the K split may be lower.  ptr_align is the smallest alignment in bytes shared by A and
  * B (pass 16 or more when they come from a device allocator). */
 int qm_select_config(int m, int n, int k, int ptr_align);
+/* The same for every form of the call: has_workspace = 0 gives what qm_gemm_i4 / qm_gemm_i4_cfg
+ * (QM_CFG_AUTO) run, which never split K through a workspace; scaled = 1 the choice of the
+ * qm_gemm_i4_scaled* forms. */
+int qm_select_config_ex(int m, int n, int k, int ptr_align, int has_workspace, int scaled);
 
 /* Introspection of the compiled-in configurations (the counterpart of the
  * KernelConfig instances, configs.cu:1-17). */

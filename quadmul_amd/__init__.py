@@ -23,7 +23,7 @@ import torch
 __all__ = [
     "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "gemm_static", "gemm_scaled", "pack_int4", "unpack_int4",
     "config_has_scaled", "quantize_pack",
-    "num_configs", "config_name", "config_names", "config_id", "select_config", "config_supports",
+    "num_configs", "config_name", "config_names", "config_id", "select_config", "select_config_ex", "config_supports",
     "CFG_AUTO", "version",
 ]
 
@@ -35,7 +35,7 @@ CFG_AUTO = -1
 #: every symbol include/qm_abi.h declares
 ABI_SYMBOLS = (
     "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled",
-    "qm_gemm_i4_ws", "qm_gemm_i4_static", "qm_gemm_i4_scaled_ws", "qm_gemm_workspace_bytes", "qm_quantize_pack_i4", "qm_select_config", "qm_num_configs", "qm_config_name",
+    "qm_gemm_i4_ws", "qm_gemm_i4_static", "qm_gemm_i4_scaled_ws", "qm_gemm_workspace_bytes", "qm_quantize_pack_i4", "qm_select_config", "qm_select_config_ex", "qm_num_configs", "qm_config_name",
     "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version",
 )
 
@@ -81,6 +81,8 @@ def library() -> ctypes.CDLL:
     lib.qm_quantize_pack_i4.restype = ci
     lib.qm_select_config.argtypes = [ci, ci, ci, ci]
     lib.qm_select_config.restype = ci
+    lib.qm_select_config_ex.argtypes = [ci, ci, ci, ci, ci, ci]
+    lib.qm_select_config_ex.restype = ci
     lib.qm_num_configs.argtypes = []
     lib.qm_num_configs.restype = ci
     lib.qm_config_name.argtypes = [ci]
@@ -324,6 +326,14 @@ def select_config(m: int, n: int, k: int, ptr_align: int = 256) -> int:
     v = int(library().qm_select_config(m, n, k, ptr_align))
     if v < 0:
         _check(v, "qm_select_config")
+    return v
+
+
+def select_config_ex(m: int, n: int, k: int, ptr_align: int = 256, workspace: bool = True, scaled: bool = False) -> int:
+    """The choice for any form of the call: with or without a workspace, int32 or scaled output."""
+    v = int(library().qm_select_config_ex(m, n, k, ptr_align, 1 if workspace else 0, 1 if scaled else 0))
+    if v < 0:
+        _check(v, "qm_select_config_ex")
     return v
 
 

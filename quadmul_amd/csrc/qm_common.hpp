@@ -85,6 +85,19 @@ __device__ __forceinline__ void x16_expand(const v4i q, v4i &even, v4i &odd)
     odd.x = x16_odd(q.x);   odd.y = x16_odd(q.y);   odd.z = x16_odd(q.z);   odd.w = x16_odd(q.w);
 }
 
+// The same in 10 instructions instead of 12: one 64-bit shift per pair of dwords (the nibble
+// that crosses into the upper dword lands in a low nibble and is masked away with the rest).
+__device__ __forceinline__ void x16_expand_pairs(const v4i q, v4i &even, v4i &odd)
+{
+    const v2i lo = {q.x, q.y}, hi = {q.z, q.w};
+    v2i slo, shi;
+    asm("v_lshlrev_b64 %0, 4, %1" : "=v"(slo) : "v"(lo));
+    asm("v_lshlrev_b64 %0, 4, %1" : "=v"(shi) : "v"(hi));
+    even.x = (int)((uint32_t)slo.x & 0xF0F0F0F0u); even.y = (int)((uint32_t)slo.y & 0xF0F0F0F0u);
+    even.z = (int)((uint32_t)shi.x & 0xF0F0F0F0u); even.w = (int)((uint32_t)shi.y & 0xF0F0F0F0u);
+    odd.x = x16_odd(q.x); odd.y = x16_odd(q.y); odd.z = x16_odd(q.z); odd.w = x16_odd(q.w);
+}
+
 // D(16x16) += S0(16x64) * S1(64x16), int8 in, int32 out.  Lane l supplies row
 // l%16 of S0 / column l%16 of S1 for the 16 k-values of group l/16, and owns
 // D[4*(l/16) + r][l%16] in register r.

@@ -11,6 +11,7 @@
 #include "../../include/qm_abi.h"
 #include "qm_launch.hpp"
 #include "qm_skinny.hpp"
+#include "qm_skinny_dma.hpp"
 #include "qm_aux.hpp"
 
 #define QM_EXPORT extern "C" __attribute__((visibility("default")))
@@ -48,6 +49,52 @@ static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int)
 }
 #define QM_DOT(MR, FN, NW, U) \
     hipError_t QM_DOT_FN(MR, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_dot<DotCfg<MR, FN, NW, U>>(p, s, gm); }
+template <class Cfg>
+static hipError_t launch_skinny_dma(const GemmArgs &p, hipStream_t stream, int)
+{
+    static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
+    const hipError_t e = ensure_dynamic_lds(&gemm_skinny_dma_kernel<Cfg>, Cfg::LDS_BYTES, lds_ok);
+    if (e != hipSuccess) return e;
+    const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
+    gemm_skinny_dma_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p);
+    return hipGetLastError();
+}
+// Compute units of the current device (asked once per device).
+static hipError_t device_cus(int *cus)
+{
+    static std::atomic<int> cached[QM_MAX_DEVICES] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= QM_MAX_DEVICES) return hipErrorInvalidDevice;
+    int n = cached[dev].load(std::memory_order_acquire);
+    if (n == 0) {
+        e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return e;
+        if (n < 1) n = 1;
+        cached[dev].store(n, std::memory_order_release);
+    }
+    *cus = n;
+    return hipSuccess;
+}
+template <class Cfg>
+static hipError_t launch_skinny_stream_dma(const GemmArgs &p, hipStream_t stream, int)
+{
+    static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
+    hipError_t e = ensure_dynamic_lds(&gemm_skinny_stream_dma_kernel<Cfg>, Cfg::LDS_BYTES, lds_ok);
+    if (e != hipSuccess) return e;
+    int cus = 0;
+    e = device_cus(&cus);
+    if (e != hipSuccess) return e;
+    const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
+    const int resident = cus * (160 * 1024 / Cfg::LDS_BYTES);  // workgroups the device holds at once (the LDS decides)
+    gemm_skinny_stream_dma_kernel<Cfg><<<dim3(blocks < resident ? blocks : resident), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, blocks);
+    return hipGetLastError();
+}
+#define QM_SKINNYP(FM, FN, NW, D, R) \
+    hipError_t QM_SKINNYP_FN(FM, FN, NW, D, R)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny_stream_dma<SkinnyStreamCfg<FM, FN, NW, D, R>>(p, s, gm); }
+#define QM_SKINNYD(FM, FN, NW, D) \
+    hipError_t QM_SKINNYD_FN(FM, FN, NW, D)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny_dma<SkinnyDmaCfg<FM, FN, NW, D>>(p, s, gm); }
 #include "qm_configs.inc"
 
 }  // namespace qm
@@ -409,6 +456,18 @@ QM_EXPORT int qm_select_config(int m, int n, int k, int ptr_align)
 {
     if (m < 1 || n < 1 || k < 2 || (k & 1)) return QM_ERR_SHAPE;
     const Choice ch = select_config(m, n, k, ptr_align, true);
+    return ch.cfg | (ch.group_m << 16) | (ch.ksplit << 24) | (ch.spread << 30);
+}
+
+QM_EXPORT int qm_select_config_ex(int m, int n, int k, int ptr_align, int has_workspace, int scaled)
+{
+    if (m < 1 || n < 1 || k < 2 || (k & 1)) return QM_ERR_SHAPE;
+    Choice ch = scaled ? select_scaled(m, n, k, ptr_align, has_workspace != 0) : select_config(m, n, k, ptr_align, has_workspace != 0);
+    if (scaled && ch.ksplit > 1 && !has_workspace) {
+        // as run_gemm: partial sums cannot meet in a rounded output
+        ch = select_scaled(m, n, k, ptr_align, false);
+        ch.ksplit = 1;
+    }
     return ch.cfg | (ch.group_m << 16) | (ch.ksplit << 24) | (ch.spread << 30);
 }
 

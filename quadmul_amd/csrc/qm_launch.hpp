@@ -47,6 +47,8 @@ inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, std::atomic<bo
 
 #define QM_SKINNY_FN(FM, FN, NW, U) qm_launch_skinny_##FM##_##FN##_##NW##_##U
 #define QM_DOT_FN(MR, FN, NW, U) qm_launch_dot_##MR##_##FN##_##NW##_##U
+#define QM_SKINNYD_FN(FM, FN, NW, D) qm_launch_skinnyd_##FM##_##FN##_##NW##_##D
+#define QM_SKINNYP_FN(FM, FN, NW, D, R) qm_launch_skinnyp_##FM##_##FN##_##NW##_##D##_##R
 #define QM_TILE16_FN(BM, BN, WGM, WGN, ST, OCC) qm_launch_tile16_##BM##_##BN##_##WGM##_##WGN##_##ST##_##OCC
 #define QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC) qm_launch_tile16s_##BM##_##BN##_##WGM##_##WGN##_##ST##_##OCC
 
@@ -54,6 +56,8 @@ inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, std::atomic<bo
 #define QM_TILE16S(tu, BM, BN, WGM, WGN, ST, OCC) hipError_t QM_TILE16S_FN(BM, BN, WGM, WGN, ST, OCC)(const GemmArgs &, hipStream_t, int);
 #define QM_SKINNY(FM, FN, NW, U) hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &, hipStream_t, int);
 #define QM_DOT(MR, FN, NW, U) hipError_t QM_DOT_FN(MR, FN, NW, U)(const GemmArgs &, hipStream_t, int);
+#define QM_SKINNYD(FM, FN, NW, D) hipError_t QM_SKINNYD_FN(FM, FN, NW, D)(const GemmArgs &, hipStream_t, int);
+#define QM_SKINNYP(FM, FN, NW, D, R) hipError_t QM_SKINNYP_FN(FM, FN, NW, D, R)(const GemmArgs &, hipStream_t, int);
 #include "qm_configs.inc"
 
 }  // namespace qm

@@ -62,18 +62,21 @@ __global__ void __launch_bounds__(256) mfma_issue_kernel(uint64_t *out, int iter
 
 __global__ void empty_kernel() {}
 
-__global__ void __launch_bounds__(256) read_kernel(const v4i *src, size_t n16, int *sink)
+// (launched with 256 or 1024 threads per workgroup and any amount of dynamic LDS, which it
+// does not touch: the launch shape is part of what is measured)
+__global__ void __launch_bounds__(1024) read_kernel(const v4i *src, size_t n16, int *sink)
 {
+    extern __shared__ __align__(16) uint8_t unused_lds[];
     v4i acc = {0, 0, 0, 0};
-    const size_t stride = (size_t)gridDim.x * 256 * 4;
-    for (size_t i = (size_t)blockIdx.x * 256 * 4 + threadIdx.x; i < n16; i += stride) {
+    const size_t per = (size_t)blockDim.x * 4, stride = (size_t)gridDim.x * per;
+    for (size_t i = (size_t)blockIdx.x * per + threadIdx.x; i < n16; i += stride) {
         v4i v[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = i + u * 256 < n16 ? __builtin_nontemporal_load(src + i + u * 256) : v4i{0, 0, 0, 0};
+        for (int u = 0; u < 4; ++u) v[u] = i + u * blockDim.x < n16 ? __builtin_nontemporal_load(src + i + u * blockDim.x) : v4i{0, 0, 0, 0};
 #pragma unroll
         for (int u = 0; u < 4; ++u) acc ^= v[u];
     }
-    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5A5A5A5B) *sink = 1;  // (practically never: keeps the loads)
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x5A5A5A5B) *sink = 1 + (int)(uintptr_t)unused_lds;  // (practically never: keeps the loads)
 }
 
 }  // namespace
@@ -97,9 +100,16 @@ QM_PROBE_EXPORT int qm_probe_empty(void *stream)
 }
 
 // `src`: 16-byte aligned device memory of `bytes` bytes (a multiple of 16); `sink`: one int.
-QM_PROBE_EXPORT int qm_probe_read(const void *src, size_t bytes, void *sink, int blocks, void *stream)
+// `threads` per workgroup: 64 .. 1024; `lds_bytes` of dynamic LDS per workgroup (untouched).
+QM_PROBE_EXPORT int qm_probe_read(const void *src, size_t bytes, void *sink, int blocks, int threads, int lds_bytes, void *stream)
 {
-    if (!src || !sink || (bytes & 15) || ((uintptr_t)src & 15) || blocks < 1) return -1;
-    read_kernel<<<dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(static_cast<const v4i *>(src), bytes / 16, static_cast<int *>(sink));
+    if (!src || !sink || (bytes & 15) || ((uintptr_t)src & 15) || blocks < 1 || threads < 64 || threads > 1024 || (threads & 63) || lds_bytes < 0 ||
+        lds_bytes > 160 * 1024)
+        return -1;
+    if (lds_bytes > 64 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&read_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return (int)e;
+    }
+    read_kernel<<<dim3(blocks), dim3(threads), lds_bytes, reinterpret_cast<hipStream_t>(stream)>>>(static_cast<const v4i *>(src), bytes / 16, static_cast<int *>(sink));
     return (int)hipGetLastError();
 }

@@ -38,7 +38,7 @@ def library() -> ctypes.CDLL:
         lib.qm_probe_mfma_issue.restype = ctypes.c_double
         lib.qm_probe_empty.argtypes = [vp]
         lib.qm_probe_empty.restype = ci
-        lib.qm_probe_read.argtypes = [vp, ctypes.c_size_t, vp, ci, vp]
+        lib.qm_probe_read.argtypes = [vp, ctypes.c_size_t, vp, ci, ci, ci, vp]
         lib.qm_probe_read.restype = ci
         _lib = lib
     return _lib
@@ -102,7 +102,7 @@ def mfma_issue_peak(seconds: float = 0.6, blocks_per_cu: int = 1):
     return res
 
 
-def launch_floor(read_bytes: int = 8 << 20, launches: int = 200, replays: int = 5):
+def launch_floor(read_bytes: int = 8 << 20, launches: int = 200, replays: int = 5, blocks: int = 512, threads: int = 256, lds_bytes: int = 0):
     """us per launch, inside a graph of back-to-back launches (median of the replays), of an
     empty kernel, of a kernel that reads `read_bytes` again and again from the same buffer
     (cache-fed) and of the same kernel rotating over copies that exceed the 256 MiB
@@ -145,10 +145,10 @@ def launch_floor(read_bytes: int = 8 << 20, launches: int = 200, replays: int = 
             raise RuntimeError(f"probe launch failed: {rc}")
 
     empty = timed(lambda i: chk(lib.qm_probe_empty(st(i))), launches)
-    hot = timed(lambda i: chk(lib.qm_probe_read(bufs[0].data_ptr(), read_bytes, sink.data_ptr(), 512, st(i))), launches)
-    cold = timed(lambda i: chk(lib.qm_probe_read(bufs[i % ncopies].data_ptr(), read_bytes, sink.data_ptr(), 512, st(i))), 5 * ncopies)
+    hot = timed(lambda i: chk(lib.qm_probe_read(bufs[0].data_ptr(), read_bytes, sink.data_ptr(), blocks, threads, lds_bytes, st(i))), launches)
+    cold = timed(lambda i: chk(lib.qm_probe_read(bufs[i % ncopies].data_ptr(), read_bytes, sink.data_ptr(), blocks, threads, lds_bytes, st(i))), 5 * ncopies)
     return {"empty_kernel_us": round(empty, 3), "read_only_us_cache_fed": round(hot, 3), "read_only_us_hbm_fed": round(cold, 3),
-            "read_bytes": read_bytes, "read_only_gbs_hbm_fed": round(read_bytes / cold / 1e3, 1),
+            "read_bytes": read_bytes, "read_launch": f"{blocks} workgroups x {threads} threads, {lds_bytes} bytes of LDS each", "read_only_gbs_hbm_fed": round(read_bytes / cold / 1e3, 1),
             "method": f"per launch inside a HIP graph of back-to-back launches, median of {replays} replays; "
                       f"HBM-fed: rotating over {ncopies} buffers (> 256 MiB)"}
 

@@ -149,18 +149,39 @@ def test_selection_rules():
     assert name(4096, 4096, 4096).startswith("q")
     assert name(4096, 4096, 4096 + 32).startswith("q")  # K % 32 == 0: the pipelined kernel with a short last K-step
     assert name(4096, 4096, 96) == "generic"            # a single short K-step: nothing for the pipelined kernel to overlap it with
-    for m in (16, 64):
-        assert name(m, 4096, 4096).startswith("s"), m
-    assert name(1, 4096, 4096).startswith("v") and name(2, 5120, 5120).startswith("v")   # dot-product kernel
-    # up to 32 rows: the skinny kernel whatever N and K; 33..64 rows: four row blocks while the
-    # 64-row tiles number one per CU at most, beyond that whichever the cost model prices lower
-    assert name(9, 28672, 14336) == "s1x1_w16_u2" and name(32, 11008, 4096) == "s2x1_w8_u4" and name(24, 4096, 8192) == "s2x1_w16_u2"
-    assert name(40, 11008, 14336) == "s4x1_w8_u2" and name(64, 14336, 4096) == "s4x1_w16_u2" and name(64, 4096, 4096) == "s4x1_w16_u1"
+    # up to 64 rows: the wave-level split-K kernels; 3..16 rows stream their operands global ->
+    # LDS, with a persistent grid and A resident in registers ("p") while the waves hold all of
+    # K, the plain form ("d") beyond
+    assert name(16, 4096, 4096) == "p1x1_w8_r2k2" and name(64, 4096, 4096) == "d4x1_w8_r1"
+    assert name(1, 4096, 4096) == "v1x1_w8_u4" and name(2, 5120, 5120) == "v2x1_w16_u2"   # dot-product kernel
+    assert name(1, 4096, 8192) == "v1x1_w16_u2" and name(2, 4096, 4096) == "v2x1_w8_u4"
+    assert name(9, 28672, 14336) == "d1x1_w16_r1" and name(9, 11008, 8192) == "p1x1_w16_r2k2" and name(12, 2048, 2048) == "d1x1_w16_r1"
+    assert name(3, 28672, 2048) == "p1x1_w8_r2k2" and name(16, 4096, 8192) == "d1x1_w16_r1"
+    assert name(32, 11008, 4096) == "p2x1_w8_r2k2" and name(24, 4096, 2048) == "p2x1_w16_r2k1"
+    assert name(24, 4096, 8192) == "d2x1_w16_r1" and name(32, 28672, 8192) == "s2x1_w16_u2"
+    assert name(40, 4096, 14336) == "d4x1_w8_r1" and name(64, 11008, 4096) == "q64x64_w2x2_s8o2"
+    # a persistent "p" configuration only takes the K its waves hold in registers
+    pk = qm.config_id("p1x1_w8_r2k2")
+    assert qm.config_supports(pk, 16, 4096, 4096) and not qm.config_supports(pk, 16, 4096, 4096 + 32) and not qm.config_supports(pk, 17, 4096, 4096)
     assert name(64, 28672, 14336).startswith("q")
     # few tiles, long K: the pipelined kernel with K split over several workgroups per tile
     code = qm.select_config(128, 8192, 28672)
     assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
     assert (qm.select_config(8192, 8192, 8192) >> 24) & 0x3F == 1
+    # ... which the table's rows were measured with: without a workspace (the plain 7-argument
+    # call) the cost model decides, and keeps a split only where it is priced below none
+    for (m, n, k) in [(128, 10240, 8192), (256, 4096, 14336), (512, 8192, 28672), (128, 8192, 28672)]:
+        with_ws, without = qm.select_config_ex(m, n, k, workspace=True), qm.select_config_ex(m, n, k, workspace=False)
+        assert (with_ws >> 24) & 0x3F > 1 and with_ws == qm.select_config(m, n, k)
+        assert qm.config_name(without & 0xFFFF).startswith("q")
+        if k <= 8192:
+            assert (without >> 24) & 0x3F == 1, (m, n, k)   # atomics lose at this K (measured)
+    # scaled output, no workspace, long K with a short last K-step: a pipelined configuration
+    # that has the output form, never the generic kernel
+    for (m, n, k) in [(256, 256, 28704), (128, 8192, 28672 + 32), (512, 4096, 14336 + 96)]:
+        code = qm.select_config_ex(m, n, k, workspace=False, scaled=True)
+        assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F == 1, (m, n, k)
+        assert qm.config_has_scaled(code & 0xFFFF)
     assert name(100, 100, 30) == "generic"          # K % 32 != 0: no 16-byte chunks
     assert name(128, 128, 4096, 4) == "generic"     # operands not 16-byte aligned
     assert name(128, 128, 262144) == "generic"      # beyond the exact range of the x16 widening

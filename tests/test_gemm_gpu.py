@@ -648,3 +648,44 @@ def test_skinny_kernel_walking_over_column_blocks(oracle_mod, shape):
         assert np.array_equal(d_d.view(torch.int16).cpu().numpy().view(np.uint16), want16), name
         ran += 1
     assert ran >= 2
+
+
+@pytest.mark.parametrize("shape", [(16, 9000, 4096), (3, 8210, 1024 + 32), (30, 4100, 2048 + 96), (13, 5000, 8192), (16, 300, 14336 + 64),
+                                   (50, 4200, 4096 + 32), (7, 33, 32), (16, 16, 65536)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_skinny_kernels_streaming_global_to_lds(oracle_mod, shape):
+    """The skinny kernels whose operands go global -> LDS directly ("d": one workgroup per
+    column block, a ring of runs per wave refilled over a long K; "p": a persistent grid
+    walking over more column blocks than the device holds workgroups, A resident in
+    registers): ragged N, short last runs of K (K % 256 = 32, 64, 96), K from one run to 256
+    runs per row.  Every such configuration that takes the shape, int32 and scaled output,
+    against the oracle; the extremes in closed form."""
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 6700 + n + k)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    want = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    a_d, b_d = ap.to(DEV), bp.to(DEV)
+    g = torch.Generator().manual_seed(SEED_BASE + 6800 + n)
+    rs, cs = torch.rand(m, generator=g) * 0.01 + 0.001, torch.rand(n, generator=g) + 0.5
+    want16 = oracle_mod.scale_round16(want, rs.numpy(), cs.numpy(), oracle_mod.OUT_F16)
+    lo_a = pack_cpu(torch.full((m, k), -8, dtype=torch.int8))
+    lo_b, hi_b = pack_cpu(torch.full((n, k), -8, dtype=torch.int8)), pack_cpu(torch.full((n, k), 7, dtype=torch.int8))
+    ran = set()
+    for cfg, name in enumerate(qm.config_names()):
+        if name[0] not in "dp" or not qm.config_supports(cfg, m, n, k):
+            continue
+        c_d = poisoned_c(m, n, DEV)
+        qm.gemm_cfg(a_d, b_d, c_d, m, n, k, cfg)
+        d_d = torch.zeros((m, n), dtype=torch.float16, device=DEV)
+        qm.gemm_scaled(a_d, b_d, d_d, m, n, k, rs.to(DEV), cs.to(DEV), cfg)
+        torch.cuda.synchronize()
+        bad = oracle_mod.compare(c_d.cpu().numpy(), want)
+        assert bad == -1, f"{name}: first mismatch at flat index {bad}"
+        assert np.array_equal(d_d.view(torch.int16).cpu().numpy().view(np.uint16), want16), name
+        if k <= 28672:
+            assert (run_gemm(lo_a, lo_b, m, n, k, cfg) == 64 * k).all(), name
+            assert (run_gemm(lo_a, hi_b, m, n, k, cfg) == -56 * k).all(), name
+        ran.add(name[0])
+    assert "d" in ran and (k > 8192 or m > 32 or "p" in ran), ran
+    if m > 2:
+        assert qm.config_name(qm.select_config(m, n, k) & 0xFFFF)[0] in "dp"
