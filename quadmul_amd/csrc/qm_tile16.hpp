@@ -432,6 +432,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     const uint32_t lane_row = ((uint32_t)(wm * Cfg::WM + (lane >> 4)) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + (lane & 15) * 4)) * (uint32_t)ESZ;
     uint8_t *const xp = smem + Cfg::RING_BYTES + wave * Cfg::XPOSE_BYTES;
     const int xp_wr = r * Cfg::XPOSE_PITCH + g * 16, xp_rd = (lane >> 4) * Cfg::XPOSE_PITCH + (lane & 15) * 16;
+    const uint32_t xp_wr_lds = lds0 + Cfg::RING_BYTES + wave * Cfg::XPOSE_BYTES + xp_wr;  // the same as an LDS address
     v4i xr[4];
     // Whole tile, through the LDS: part t = 0..7 of blocks (ib, 4*grp .. 4*grp+3), one part per
     // MFMA slot.  Parts 0..3 write one block each; the read-back of row quartet k and its
@@ -445,11 +446,25 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         auto store_rows = [&](auto k_) __attribute__((always_inline)) {
             constexpr int k = decltype(k_)::value;
             char *const at = tile_c + ((size_t)(ib * 16 + 4 * k) * p.N + grp * 64) * ESZ;  // wave-uniform
-            if constexpr (OUT == OUT_I32) *reinterpret_cast<v4i *>(at + lane_row) = xr[k];
-            else *reinterpret_cast<v2i *>(at + lane_row) = pack16(xr[k]);
+            if constexpr (OUT == OUT_I32) {
+                v4i v = xr[k];
+                v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
+                *reinterpret_cast<v4i *>(at + lane_row) = v;
+            } else {
+                *reinterpret_cast<v2i *>(at + lane_row) = pack16(xr[k]);
+            }
         };
-        if constexpr (t < 4)
-            *reinterpret_cast<v4i *>(xp + xp_wr + 64 * t) = take_block(ib_, std::integral_constant<int, 4 * grp + t>{});
+        if constexpr (t < 4) {
+            if constexpr (OUT == OUT_I32) {
+                // int32: the block goes to the LDS area as it is -- 256 x the result, straight
+                // from its accumulator registers (a DS instruction takes them as data) -- and is
+                // cleared behind; the factor is dropped after the read-back, in row order
+                asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(xp_wr_lds), "a"(acc[ib][4 * grp + t]), "n"(64 * t) : "memory");
+                mfma16_zero(acc[ib][4 * grp + t], zero4);
+            } else {
+                *reinterpret_cast<v4i *>(xp + xp_wr + 64 * t) = take_block(ib_, std::integral_constant<int, 4 * grp + t>{});
+            }
+        }
         if constexpr (t == 3) read_back(std::integral_constant<int, 0>{});
         if constexpr (t == 4) read_back(std::integral_constant<int, 1>{});
         if constexpr (t == 5) { read_back(std::integral_constant<int, 2>{}); store_rows(std::integral_constant<int, 0>{}); }
