@@ -184,7 +184,19 @@ int qm_unpack_i4(const void *src_packed, void *dst_i8, int rows, int k, void *st
 #define QM_IN_F32  3
 int qm_quantize_pack_i4(const void *x, int in_dtype, void *dst_packed, float *scales, int rows, int k, void *stream);
 
-/* Diagnostics. */
+/*
+ * Optional: everything a first launch on the current device would otherwise do once -- the
+ * LDS size attribute and the residency query of every kernel, the address of the library's
+ * scratch array -- without launching anything.  No counterpart in the reference (its
+ * launch_igemm, kernel.cu:268-289, needs no set-up: 32 KB of shared memory at most).  First
+ * launches do this by themselves, under HIP graph capture too; a caller that wants no
+ * runtime queries inside a capture or a latency-critical first call makes this call first,
+ * once per device, with that device current.
+ */
+int qm_init(void);
+
+/* Diagnostics.  qm_version names the compiler the library was built with: the kernels
+ * manage matrix-core hazards by hand, so a result is validated for that compiler. */
 const char *qm_status_string(int status);
 int         qm_last_hip_error(void);      /* hipError_t of the last failed launch on this thread */
 const char *qm_version(void);

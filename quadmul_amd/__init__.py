@@ -24,7 +24,7 @@ __all__ = [
     "QuadmulError", "library", "library_path", "gemm", "gemm_cfg", "gemm_static", "gemm_scaled", "pack_int4", "unpack_int4",
     "config_has_scaled", "quantize_pack",
     "num_configs", "config_name", "config_names", "config_id", "select_config", "select_config_ex", "config_supports",
-    "CFG_AUTO", "version",
+    "CFG_AUTO", "version", "init",
 ]
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
@@ -36,7 +36,7 @@ CFG_AUTO = -1
 ABI_SYMBOLS = (
     "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled",
     "qm_gemm_i4_ws", "qm_gemm_i4_static", "qm_gemm_i4_scaled_ws", "qm_gemm_workspace_bytes", "qm_quantize_pack_i4", "qm_select_config", "qm_select_config_ex", "qm_num_configs", "qm_config_name",
-    "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version",
+    "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version", "qm_init",
 )
 
 
@@ -97,6 +97,8 @@ def library() -> ctypes.CDLL:
     lib.qm_status_string.restype = ctypes.c_char_p
     lib.qm_last_hip_error.argtypes = []
     lib.qm_last_hip_error.restype = ci
+    lib.qm_init.argtypes = []
+    lib.qm_init.restype = ci
     lib.qm_version.argtypes = []
     lib.qm_version.restype = ctypes.c_char_p
     _lib = lib
@@ -297,6 +299,13 @@ def unpack_int4(packed: torch.Tensor) -> torch.Tensor:
     lo = torch.where(lo > 7, lo - 16, lo)
     hi = torch.where(hi > 7, hi - 16, hi)
     return torch.stack((lo, hi), dim=2).reshape(rows, 2 * half).to(torch.int8)
+
+
+def init(device=None) -> None:
+    """Every kernel's one-off set-up on ``device`` (default: the current one) without launching
+    anything; optional -- first launches do it by themselves."""
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        _check(library().qm_init(), "qm_init")
 
 
 def num_configs() -> int:

@@ -43,6 +43,25 @@ def ext_path() -> str:
     return os.path.join(ROOT, "quadmul" + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
+# The compilers the full GPU suite has passed with.  The kernels order matrix-core
+# instructions and their hazards by hand inside asm statements; another compiler may schedule
+# the code around them differently, so a build with one is flagged until the suite has been
+# run on it (tests/ -m gpu is the gate).
+VALIDATED_COMPILERS = ("HIP version: 7.2",)
+
+
+def compiler_version() -> str:
+    try:
+        out = subprocess.run([HIPCC, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True).stdout
+    except OSError:
+        return "unknown compiler"
+    lines = [l.strip() for l in out.splitlines() if l.strip()]
+    hip = next((l for l in lines if l.startswith("HIP version")), "")
+    clang = next((l for l in lines if "clang version" in l), "")
+    clang = clang.split("(")[0].strip()
+    return "; ".join(x for x in (hip, clang) if x) or "unknown compiler"
+
+
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
@@ -54,7 +73,11 @@ def _run(cmd):
 def build_lib(jobs: int = 8, verbose: bool = False) -> str:
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
-    units = [("qm_dispatch.o", ["-c", os.path.join(CSRC, "qm_dispatch.hip")])]
+    ver = compiler_version()
+    if not any(ver.startswith(v) for v in VALIDATED_COMPILERS):
+        print(f"quadmul_amd.build: WARNING: building with {ver!r}, which the GPU test-suite has not been run with "
+              f"(validated: {', '.join(VALIDATED_COMPILERS)}); run `pytest tests -m gpu` before trusting results", file=sys.stderr)
+    units = [("qm_dispatch.o", [f'-DQM_COMPILER_VERSION="{ver}"', "-c", os.path.join(CSRC, "qm_dispatch.hip")])]
     for tu in range(N_TILE_TUS):
         units.append((f"qm_tile_inst_{tu}.o", [f"-DQM_TU={tu}", "-c", os.path.join(CSRC, "qm_tile_inst.hip")]))
     objs = [os.path.join(OBJDIR, name) for name, _ in units]

@@ -22,8 +22,9 @@ namespace qm {
 // Launchers of the skinny and dot kernels
 // --------------------------------------------------------------------------
 template <class Cfg>
-static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
+static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int opt)
 {
+    if (opt & QM_OPT_PREPARE) return hipSuccess;  // static LDS, nothing to set up
     const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
     // More column blocks than two workgroups per CU can hold at once, and K within one turn
     // of the waves: workgroups that walk over several blocks each, evenly.
@@ -41,8 +42,9 @@ static hipError_t launch_skinny(const GemmArgs &p, hipStream_t stream, int)
 #define QM_SKINNY(FM, FN, NW, U) \
     hipError_t QM_SKINNY_FN(FM, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_skinny<SkinnyCfg<FM, FN, NW, U>>(p, s, gm); }
 template <class Cfg>
-static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int)
+static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int opt)
 {
+    if (opt & QM_OPT_PREPARE) return hipSuccess;
     const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
     gemm_dot_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), 0, stream>>>(p);
     return hipGetLastError();
@@ -50,11 +52,12 @@ static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int)
 #define QM_DOT(MR, FN, NW, U) \
     hipError_t QM_DOT_FN(MR, FN, NW, U)(const GemmArgs &p, hipStream_t s, int gm) { return launch_dot<DotCfg<MR, FN, NW, U>>(p, s, gm); }
 template <class Cfg>
-static hipError_t launch_skinny_dma(const GemmArgs &p, hipStream_t stream, int)
+static hipError_t launch_skinny_dma(const GemmArgs &p, hipStream_t stream, int opt)
 {
     static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
     const hipError_t e = ensure_dynamic_lds(&gemm_skinny_dma_kernel<Cfg>, Cfg::LDS_BYTES, lds_ok);
     if (e != hipSuccess) return e;
+    if (opt & QM_OPT_PREPARE) return hipSuccess;
     const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
     gemm_skinny_dma_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p);
     return hipGetLastError();
@@ -78,7 +81,7 @@ static hipError_t device_cus(int *cus)
     return hipSuccess;
 }
 template <class Cfg>
-static hipError_t launch_skinny_stream_dma(const GemmArgs &p, hipStream_t stream, int)
+static hipError_t launch_skinny_stream_dma(const GemmArgs &p, hipStream_t stream, int opt)
 {
     static std::atomic<bool> lds_ok[QM_MAX_DEVICES] = {};
     hipError_t e = ensure_dynamic_lds(&gemm_skinny_stream_dma_kernel<Cfg>, Cfg::LDS_BYTES, lds_ok);
@@ -86,6 +89,7 @@ static hipError_t launch_skinny_stream_dma(const GemmArgs &p, hipStream_t stream
     int cus = 0;
     e = device_cus(&cus);
     if (e != hipSuccess) return e;
+    if (opt & QM_OPT_PREPARE) return hipSuccess;
     const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
     const int resident = cus * (160 * 1024 / Cfg::LDS_BYTES);  // workgroups the device holds at once (the LDS decides)
     gemm_skinny_stream_dma_kernel<Cfg><<<dim3(blocks < resident ? blocks : resident), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, blocks);
@@ -369,6 +373,28 @@ static hipError_t static_scratch(void **out)
     return hipSuccess;
 }
 
+// Every one-off set-up a first launch on the current device would otherwise do.
+QM_EXPORT int qm_init(void)
+{
+    GemmArgs p{nullptr, nullptr, nullptr, 256, 256, 256};
+    for (int id = 0; id < g_num_configs; ++id) {
+        if (g_configs[id].kind == KIND_GENERIC) continue;
+        for (const int k : {256, 256 + 32}) {   // the kernel for whole K-steps and the one with a short last step
+            p.K = k;
+            for (const int out : {(int)OUT_I32, (int)OUT_F16, (int)OUT_BF16}) {
+                const LaunchFn fn = out == OUT_I32 ? g_configs[id].launch : scaled_launcher(id);
+                if (!fn || (out != OUT_I32 && g_configs[id].kind != KIND_TILE16)) continue;
+                p.out = out;
+                const hipError_t e = fn(p, nullptr, QM_OPT_PREPARE);
+                if (e != hipSuccess) return fail_launch(e);
+            }
+        }
+    }
+    void *ws = nullptr;
+    const hipError_t e = static_scratch(&ws);
+    return e == hipSuccess ? QM_OK : fail_launch(e);
+}
+
 QM_EXPORT int qm_gemm_i4_static(const void *A, const void *B, void *C, int m, int n, int k, void *stream)
 {
     const int st = check_gemm_args(A, B, C, m, n, k);
@@ -546,4 +572,7 @@ QM_EXPORT const char *qm_status_string(int status)
 
 QM_EXPORT int qm_last_hip_error(void) { return g_last_hip_error; }
 
-QM_EXPORT const char *qm_version(void) { return "quadmul-amd 0.1 (gfx950)"; }
+#ifndef QM_COMPILER_VERSION
+#define QM_COMPILER_VERSION "unknown compiler"
+#endif
+QM_EXPORT const char *qm_version(void) { return "quadmul-amd 0.2 (gfx950; built with " QM_COMPILER_VERSION ")"; }

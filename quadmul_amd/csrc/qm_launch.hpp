@@ -10,6 +10,9 @@ namespace qm {
 typedef hipError_t (*LaunchFn)(const GemmArgs &, hipStream_t, int group_m);
 
 constexpr int QM_MAX_DEVICES = 64;
+// bit of a launcher's third argument: do the kernel's one-off set-up on the current device
+// (LDS size attribute, residency query) and return without launching
+constexpr int QM_OPT_PREPARE = 1 << 17;
 
 // K split of the pipelined kernel, normalised: kt K-steps of 128 nibbles (the last one may
 // be short); with kps steps per split only ceil(kt / kps) splits have work; and a split

@@ -10,8 +10,9 @@
 namespace qm {
 
 // opt: tile raster group height in bits 0..7, the K split in bits 8..15 (the caller has
-// zero-filled C, or given the kernel a workspace, when it is above 1) and, in bit 16, "one
-// work item per workgroup".  By
+// zero-filled C, or given the kernel a workspace, when it is above 1), in bit 16 "one
+// work item per workgroup", and in bit 17 "prepare only" (qm_init: the kernel's one-off
+// set-up on this device, no launch).  By
 // default the grid is persistent: as many workgroups as the device holds at once, each
 // running several (K split, tile) items back to back.
 // (OUT is a template parameter so that every kernel gets launcher statics of its own.)
@@ -40,6 +41,7 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
         held = g < 8 ? 8 : g;
         resident[dev].store(held, std::memory_order_release);
     }
+    if (opt & QM_OPT_PREPARE) return hipSuccess;  // the one-off set-up above was all that was asked for
     const int tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM, tiles_n = (p.N + Cfg::BN - 1) / Cfg::BN;
     int group_m = opt & 0xFF, ksplit = (opt >> 8) & 0xFF;
     if (group_m < 1) group_m = 1;

@@ -132,6 +132,11 @@ def test_workspace_sizes():
     assert qm.workspace_bytes(4096, 4096, 4162, qm.config_id("generic")) == 0   # explicit configuration: as asked
 
 
+def test_version_names_the_compiler():
+    v = qm.version()
+    assert v.startswith("quadmul-amd") and "gfx950" in v and "HIP version" in v, v
+
+
 def test_config_registry():
     names = qm.config_names()
     assert names[0] == "generic" and len(names) == len(set(names))
