@@ -171,7 +171,7 @@ static PadPlan plan_padded_k(int m, int n, int k, int ptr_align, const Choice &d
     const int kp = (k + 127) / 128 * 128;
     if (kp > QM_MAX_K_X16 || !fast_path_ok(m, n, kp, 256)) return pl;
     const long long outs = (long long)m * n;
-    if (outs * k < (1LL << 27)) return pl;
+    if (outs * kp < (1LL << 27)) return pl;  // (kp: a K below one K-step counts as the step it is padded to)
     (void)ptr_align;
     Choice ch = heuristic(m, n, kp, 256, false);
     if (g_configs[ch.cfg].kind == KIND_GENERIC) return pl;

@@ -427,6 +427,11 @@ def test_random_shapes_through_the_automatic_choice():
         name = qm.config_name(code & 0xFFFF)
         seen.add(name[0] + ("+split" if (code >> 24) & 0x3F > 1 else ""))
         assert torch.equal(c_d, want), f"{m}x{n}x{k} ({name}, ksplit {(code >> 24) & 0x3F})"
+        # nothing of 2^27 multiply-adds or more is left to the one-thread-per-element kernel:
+        # where no fast kernel takes the operands as they are, the call runs on padded copies
+        # in the workspace (which quadmul.gemm provides)
+        if name == "generic" and m * n * ((k + 127) // 128 * 128) >= 2 ** 27 and k <= 131000:
+            assert qm.workspace_bytes(m, n, k) > 0, (m, n, k)
     assert {"g", "s", "q", "q+split"} <= seen, seen
 
 
@@ -454,12 +459,13 @@ def test_dot_product_kernel_one_and_two_rows(oracle_mod, shape):
     assert oracle_mod.compare(run_gemm(ap, bp, m, n, k), want) == -1
 
 
-@pytest.mark.parametrize("shape", [(3000, 3000, 1056), (1000, 1000, 1000), (1000, 1100, 1004), (300, 5000, 4098), (2100, 4200, 96 + 2)],
+@pytest.mark.parametrize("shape", [(3000, 3000, 1056), (1000, 1000, 1000), (1000, 1100, 1004), (300, 5000, 4098), (2100, 4200, 96 + 2),
+                                   (2100, 4200, 96), (1500, 1500, 64), (4096, 4096, 32)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_k_padded_through_the_workspace(shape):
-    """Large shapes whose K is not a multiple of 32, and unaligned operands: with a workspace
-    the operands are copied with zero-padded rows and the pipelined kernel runs; without one
-    the generic kernel does.  (K % 32 == 0, first case: no copies, a short last K-step.)  Same
+    """Large shapes whose K is not a multiple of 32 or is less than one K-step, and unaligned
+    operands: with a workspace the operands are copied with zero-padded rows and the
+    pipelined kernel runs; without one the generic kernel does.  (K % 32 == 0, first case: no copies, a short last K-step.)  Same
     result, against an exact fp32 matmul."""
     import quadmul
 
@@ -469,7 +475,7 @@ def test_k_padded_through_the_workspace(shape):
     want = fp32_matmul_on_gpu(a, b)
     ap, bp = pack_cpu(a), pack_cpu(b)
     a_d, b_d = ap.to(DEV), bp.to(DEV)
-    if k % 32:
+    if k % 32 or k < 128:   # (less than one whole K-step: nothing for a short last step to follow)
         assert qm.workspace_bytes(m, n, k) >= (m + n) * ((k + 127) // 128 * 64)
     else:   # K % 32 == 0: the pipelined kernel runs it as it is, with a short last K-step
         assert qm.workspace_bytes(m, n, k) == 0 and qm.config_name(qm.select_config(m, n, k) & 0xFFFF).startswith("q")
