@@ -44,7 +44,7 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(const GemmArgs p, con
     }
     const int m = m0 + ty, n = n0 + tx;
     if (m < p.M && n < p.N) {
-        const size_t at = (size_t)m * p.N + n;
+        const size_t at = (size_t)m * c_stride(p) + n;
         if (p.out == OUT_I32) p.C[at] = sum;
         else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(sum, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
     }

@@ -28,7 +28,12 @@ struct GemmArgs {
     // launch stores its tile here, 16 bytes per lane in the order the MFMA leaves them, and a
     // second kernel adds the splits up.
     int32_t *ws = nullptr;
+    // Row stride of C in elements, 0 standing for N: set when the call computes a block of
+    // columns of a wider C (a B beyond the kernels' 32-bit offsets is cut along N).
+    int ldc = 0;
 };
+
+__device__ __forceinline__ int c_stride(const GemmArgs &p) { return p.ldc != 0 ? p.ldc : p.N; }
 
 __device__ __forceinline__ float scale_at(const float *s, int i, int n) { return (s != nullptr && i < n) ? s[i] : 1.0f; }
 

@@ -252,11 +252,23 @@ static hipError_t launch_split_with_workspace(GemmArgs p, const Choice &ch, void
 // as well, or a shape the fast kernels do not take anyway).
 static int row_block_for_large_a(int m, int n, int k, int ptr_align)
 {
+    (void)n;
     if (k < 32 || k % 32 != 0 || k > QM_MAX_K_X16 || ptr_align < 16) return 0;
     const long long kb = k / 2;
-    if ((long long)m * kb < 0x7fffffffLL || (long long)n * kb >= 0x7fffffffLL) return 0;
+    if ((long long)m * kb < 0x7fffffffLL) return 0;
     const long long rows = ((0x7fffffffLL - 1) / kb) & ~255LL;
     return rows >= 256 ? (int)rows : 0;
+}
+
+// The same for a B of 2 GiB or more (and an A that fits, or a row block of one): blocks of
+// rows of B are blocks of columns of C, which the kernels write through a row stride.
+static int col_block_for_large_b(int m, int n, int k, int ptr_align)
+{
+    if (k < 32 || k % 32 != 0 || k > QM_MAX_K_X16 || ptr_align < 16) return 0;
+    const long long kb = k / 2;
+    if ((long long)n * kb < 0x7fffffffLL || (long long)m * kb >= 0x7fffffffLL) return 0;
+    const long long cols = ((0x7fffffffLL - 1) / kb) & ~255LL;
+    return cols >= 256 ? (int)cols : 0;
 }
 
 // One GEMM call, arguments already checked (m, n >= 1, k even).  `out` is OUT_I32 with C in
@@ -264,10 +276,12 @@ static int row_block_for_large_a(int m, int n, int k, int ptr_align)
 // place: a K split whose partial sums have no workspace to meet in falls back to atomic adds
 // into a zero-filled C for int32, and is not taken at all for a rounded output.
 static int run_gemm(const void *A, const void *B, void *dst, int m, int n, int k, const float *row_scale,
-                    const float *col_scale, int out, hipStream_t s, int cfg, void *workspace, size_t workspace_bytes)
+                    const float *col_scale, int out, hipStream_t s, int cfg, void *workspace, size_t workspace_bytes, int ldc = 0)
 {
     const bool scaled = out != OUT_I32;
     const size_t cnt = (size_t)m * (size_t)n;
+    const int row_stride = ldc != 0 ? ldc : n;   // of the output, in elements
+    const bool strided = row_stride != n;        // a block of columns of a wider output
     if (k == 0) {
         if (scaled) fill_zero16_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<uint16_t *>(dst), cnt);
         else fill_zero_kernel<<<dim3(flat_grid(cnt, 256)), dim3(256), 0, s>>>(static_cast<int32_t *>(dst), cnt);
@@ -278,8 +292,17 @@ static int run_gemm(const void *A, const void *B, void *dst, int m, int n, int k
     if (const int rb = cfg == QM_CFG_AUTO ? row_block_for_large_a(m, n, k, align) : 0) {
         for (int r0 = 0; r0 < m; r0 += rb) {
             const int st = run_gemm(static_cast<const uint8_t *>(A) + (size_t)r0 * (size_t)(k / 2), B,
-                                    static_cast<uint8_t *>(dst) + (size_t)r0 * (size_t)n * (scaled ? 2 : 4), m - r0 < rb ? m - r0 : rb,
-                                    n, k, row_scale ? row_scale + r0 : nullptr, col_scale, out, s, cfg, workspace, workspace_bytes);
+                                    static_cast<uint8_t *>(dst) + (size_t)r0 * (size_t)row_stride * (scaled ? 2 : 4), m - r0 < rb ? m - r0 : rb,
+                                    n, k, row_scale ? row_scale + r0 : nullptr, col_scale, out, s, cfg, workspace, workspace_bytes, ldc);
+            if (st != QM_OK) return st;
+        }
+        return QM_OK;
+    }
+    if (const int cb = cfg == QM_CFG_AUTO ? col_block_for_large_b(m, n, k, align) : 0) {
+        for (int c0 = 0; c0 < n; c0 += cb) {
+            const int st = run_gemm(A, static_cast<const uint8_t *>(B) + (size_t)c0 * (size_t)(k / 2),
+                                    static_cast<uint8_t *>(dst) + (size_t)c0 * (scaled ? 2 : 4), m, n - c0 < cb ? n - c0 : cb, k, row_scale,
+                                    col_scale ? col_scale + c0 : nullptr, out, s, cfg, workspace, workspace_bytes, row_stride);
             if (st != QM_OK) return st;
         }
         return QM_OK;
@@ -289,8 +312,20 @@ static int run_gemm(const void *A, const void *B, void *dst, int m, int n, int k
     p.row_scale = row_scale;
     p.col_scale = col_scale;
     p.out = out;
+    p.ldc = strided ? row_stride : 0;
+    if (strided && cfg != QM_CFG_AUTO) return QM_ERR_CONFIG;
     const auto launcher = [&](int id) { return scaled ? scaled_launcher(id) : g_configs[id].launch; };
     Choice ch;
+    if (strided) {
+        // one launch straight into the wider output: no K split (its partial sums are added up
+        // into a contiguous C) and no padded copies
+        ch = scaled ? select_scaled(m, n, k, align, false) : select_config(m, n, k, align, false);
+        ch.ksplit = 1;
+        const LaunchFn launch = launcher(ch.cfg);
+        if (!launch) return QM_ERR_CONFIG;
+        const hipError_t e = launch(p, s, ch.group_m | (1 << 8) | (ch.spread << 16));
+        return e == hipSuccess ? QM_OK : fail_launch(e);
+    }
     if (cfg == QM_CFG_AUTO) {
         ch = scaled ? select_scaled(m, n, k, align, has_ws) : select_config(m, n, k, align, has_ws);
     } else {
@@ -451,6 +486,7 @@ QM_EXPORT size_t qm_gemm_workspace_bytes(int m, int n, int k, int ptr_align, int
         const size_t rest = m % rb ? qm_gemm_workspace_bytes(m % rb, n, k, ptr_align, cfg, scaled) : 0;
         return whole > rest ? whole : rest;
     }
+    if (cfg == QM_CFG_AUTO && col_block_for_large_b(m, n, k, ptr_align)) return 0;  // blocks of columns: one launch each, no workspace
     Choice ch;
     if (cfg == QM_CFG_AUTO) {
         ch = scaled ? select_scaled(m, n, k, ptr_align, true) : select_config(m, n, k, ptr_align, true);

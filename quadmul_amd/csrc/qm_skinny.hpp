@@ -186,7 +186,7 @@ gemm_skinny_kernel(const GemmArgs p)
         const int32_t s = red[blk][nl & 3][ml + 16 * (nl >> 2)];
         const int m = (blk / FN) * 16 + ml, n = n0 + (blk % FN) * 16 + nl;
         if (m < p.M && n < p.N) {
-            const size_t at = (size_t)m * p.N + n;
+            const size_t at = (size_t)m * c_stride(p) + n;
             if (p.out == OUT_I32) p.C[at] = s >> 8;
             else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s >> 8, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
         }
@@ -306,7 +306,7 @@ gemm_skinny_stream_kernel(const GemmArgs p, const int nblocks)
             *at_red = 0;
             const int m = (b / FN) * 16 + ml, n = n0 + (b % FN) * 16 + nl;
             if (m < p.M && n < p.N) {
-                const size_t at = (size_t)m * p.N + n;
+                const size_t at = (size_t)m * c_stride(p) + n;
                 if (p.out == OUT_I32) p.C[at] = s >> 8;
                 else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s >> 8, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
             }
@@ -417,7 +417,7 @@ gemm_dot_kernel(const GemmArgs p)
         const int m = idx / (FN * 16), n = n0 + idx % (FN * 16);
         if (m < p.M && n < p.N) {
             const int32_t s = (&red[0][0])[idx];
-            const size_t at = (size_t)m * p.N + n;
+            const size_t at = (size_t)m * c_stride(p) + n;
             if (p.out == OUT_I32) p.C[at] = s;
             else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
         }

@@ -208,7 +208,7 @@ gemm_skinny_dma_kernel(const GemmArgs p)
     if (ticket != NW - 1) return;
 
     // lane (r, g) of block (i, j) holds C[16 i + r][n0 + 16 j + 4 g .. + 3]
-    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & (p.out == OUT_I32 ? 15 : 7)) == 0;
+    const bool vec_ok = (c_stride(p) & 3) == 0 && ((uintptr_t)p.C & (p.out == OUT_I32 ? 15 : 7)) == 0;
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -218,10 +218,10 @@ gemm_skinny_dma_kernel(const GemmArgs p)
             for (int e = 0; e < 4; ++e) s[e] = red[((i * FN + j) * 4 + e) * 64 + lane] >> 8;
             const int m = i * 16 + r, n = n0 + j * 16 + 4 * g;
             if (m >= p.M || n >= p.N) continue;
-            const size_t at = (size_t)m * p.N + n;
+            const size_t at = (size_t)m * c_stride(p) + n;
             if (p.out == OUT_I32) {
                 if (vec_ok) {
-                    *reinterpret_cast<v4i *>(p.C + at) = s;  // n % 4 == 0 and N % 4 == 0: all four inside
+                    *reinterpret_cast<v4i *>(p.C + at) = s;  // n % 4 == 0 and N % 4 == 0 (with a row stride: N is that stride or differs from it by a multiple of 256): all four inside
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
@@ -436,7 +436,7 @@ gemm_skinny_stream_dma_kernel(const GemmArgs p, const int nblocks)
             *at_red = 0;
             const int m = (bb / FN) * 16 + ml, n = n0 + (bb % FN) * 16 + nl;
             if (m < p.M && n < p.N) {
-                const size_t at = (size_t)m * p.N + n;
+                const size_t at = (size_t)m * c_stride(p) + n;
                 if (p.out == OUT_I32) p.C[at] = s >> 8;
                 else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s >> 8, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
             }

@@ -198,8 +198,9 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // column and bottom row of tiles; or all items, when nwhole is 0), written out by the
     // guarded code after the last K-step.  A workgroup's items ascend, so it runs its whole
     // tiles first and then the rest: two loops one after the other.
-    const bool vec_ok = (p.N & 3) == 0 && ((uintptr_t)p.C & (4 * ESZ - 1)) == 0;  // 4 elements per store
-    const bool plain_c = vec_ok && ksplit == 1 && p.N < (1 << 21);
+    const int ldc = c_stride(p);  // row stride of C in elements (N, unless this call computes a block of columns of a wider C)
+    const bool vec_ok = (ldc & 3) == 0 && ((uintptr_t)p.C & (4 * ESZ - 1)) == 0;  // 4 elements per store
+    const bool plain_c = vec_ok && ksplit == 1 && ldc < (1 << 21);
     const int full_m = p.M / BM, full_n = p.N / BN;
     const int nwhole = __builtin_amdgcn_readfirstlane(plain_c ? full_m * full_n : 0);
     auto locate = [&](const int item, int &m0, int &n0, int &kt0, int &KT) __attribute__((always_inline)) {
@@ -428,8 +429,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     };
     // byte offsets of this lane from the tile's corner (32 bits are enough for the rows of one
     // tile when N is below 2^21): as the MFMA leaves a block, and as the LDS area is read back
-    const uint32_t lane_blk = ((uint32_t)(wm * Cfg::WM + r) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + g * 4)) * (uint32_t)ESZ;
-    const uint32_t lane_row = ((uint32_t)(wm * Cfg::WM + (lane >> 4)) * (uint32_t)p.N + (uint32_t)(wn * Cfg::WN + (lane & 15) * 4)) * (uint32_t)ESZ;
+    const uint32_t lane_blk = ((uint32_t)(wm * Cfg::WM + r) * (uint32_t)ldc + (uint32_t)(wn * Cfg::WN + g * 4)) * (uint32_t)ESZ;
+    const uint32_t lane_row = ((uint32_t)(wm * Cfg::WM + (lane >> 4)) * (uint32_t)ldc + (uint32_t)(wn * Cfg::WN + (lane & 15) * 4)) * (uint32_t)ESZ;
     uint8_t *const xp = smem + Cfg::RING_BYTES + wave * Cfg::XPOSE_BYTES;
     const int xp_wr = r * Cfg::XPOSE_PITCH + g * 16, xp_rd = (lane >> 4) * Cfg::XPOSE_PITCH + (lane & 15) * 16;
     const uint32_t xp_wr_lds = lds0 + Cfg::RING_BYTES + wave * Cfg::XPOSE_BYTES + xp_wr;  // the same as an LDS address
@@ -445,7 +446,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         };
         auto store_rows = [&](auto k_) __attribute__((always_inline)) {
             constexpr int k = decltype(k_)::value;
-            char *const at = tile_c + ((size_t)(ib * 16 + 4 * k) * p.N + grp * 64) * ESZ;  // wave-uniform
+            char *const at = tile_c + ((size_t)(ib * 16 + 4 * k) * ldc + grp * 64) * ESZ;  // wave-uniform
             if constexpr (OUT == OUT_I32) {
                 v4i v = xr[k];
                 v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
@@ -477,7 +478,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         if constexpr (t == 0) {
             xr[0] = take_block(ib_, j_);
         } else {
-            char *const at = tile_c + ((size_t)(ib * 16) * p.N + j * 16) * ESZ;  // wave-uniform
+            char *const at = tile_c + ((size_t)(ib * 16) * ldc + j * 16) * ESZ;  // wave-uniform
             if constexpr (OUT == OUT_I32) *reinterpret_cast<v4i *>(at + lane_blk) = xr[0];
             else *reinterpret_cast<v2i *>(at + lane_blk) = pack16(xr[0]);
         }
@@ -503,7 +504,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         const int m = (c_m0 + ib * 16) + (wm * Cfg::WM + r), n = (c_n0 + j * 16) + (wn * Cfg::WN + g * 4);
         if constexpr (OUT != OUT_I32) {
             if (m < p.M) {
-                uint16_t *drow = reinterpret_cast<uint16_t *>(p.C) + (size_t)m * p.N;
+                uint16_t *drow = reinterpret_cast<uint16_t *>(p.C) + (size_t)m * ldc;
                 const v2i o = pack16(v);
                 if (vec_ok && n + 3 < p.N) {
                     *reinterpret_cast<v2i *>(drow + n) = o;
@@ -515,7 +516,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 }
             }
         } else if (m < p.M) {
-            int32_t *crow = p.C + (size_t)m * p.N;
+            int32_t *crow = p.C + (size_t)m * ldc;
             if (ksplit > 1) {
                 // every partial accumulator is a multiple of 256, so the shifted partials add
                 // up to the shifted total; integer atomics make the order irrelevant
@@ -678,7 +679,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             asm volatile("" : "+s"(bmask));
             full = amask;
         }
-        tile_c = reinterpret_cast<char *>(p.C) + ((size_t)c_m0 * p.N + c_n0) * ESZ;
+        tile_c = reinterpret_cast<char *>(p.C) + ((size_t)c_m0 * ldc + c_n0) * ESZ;
         if constexpr (OUT == OUT_I32 && !whole) {
             // workspace slot of a K-split item: (split, tile) in the order locate() numbers them
             if (p.ws != nullptr && ksplit > 1)

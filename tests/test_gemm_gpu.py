@@ -527,7 +527,8 @@ def test_short_last_k_step_on_every_pipelined_config(oracle_mod, k):
 
 def test_operands_of_two_gib_and_more(oracle_mod):
     """An A of 2 GiB or more is cut into row blocks that fit the fast kernels' 32-bit row
-    offsets; a B that large goes to the generic kernel (64-bit offsets).  Every row is compared
+    offsets, a B that large into blocks of its rows (blocks of columns of C, written through a
+    row stride).  Every row is compared
     with the library's own result on slices below the limit (paths the other tests pin against
     the oracle), and the rows either side of the block boundary and the last rows with the
     oracle itself.  Packed bytes are drawn on the GPU: any byte is two valid nibbles."""
@@ -564,20 +565,38 @@ def test_operands_of_two_gib_and_more(oracle_mod):
         ref = oracle_mod.scale_round16(want[r0:r0 + 40].cpu().numpy(), rs[r0:r0 + 40].cpu().numpy(), cs.cpu().numpy(), oracle_mod.OUT_F16)
         assert np.array_equal(d_d[r0:r0 + 40].cpu().numpy().view(np.uint16), ref)
     del a_d, want, c_d, d_d
-    # --- large B ---
-    m, n = 8, (1 << 20) + 20
-    a_d = torch.randint(-128, 128, (m, kb), dtype=torch.int8, device=DEV, generator=g)
+    # --- large B: cut into blocks of its rows, i.e. blocks of columns of C, which the kernels
+    # write through a row stride; a skinny shape and one for the pipelined tile kernel ---
+    n = (1 << 20) + 20
+    assert n * kb >= 2 ** 31
     b_d = torch.randint(-128, 128, (n, kb), dtype=torch.int8, device=DEV, generator=g)
-    assert qm.config_name(qm.select_config(m, n, k) & 0xFFFF) == "generic"
-    c_d = poisoned_c(m, n, DEV)
-    quadmul.gemm(a_d, b_d, c_d, m, n, k)
-    for c0 in range(0, n, 262144):
-        cols = min(262144, n - c0)
-        part = torch.empty((m, cols), dtype=torch.int32, device=DEV)
-        qm.gemm(a_d, b_d[c0:c0 + cols], part, m, cols, k)
-        assert torch.equal(c_d[:, c0:c0 + cols], part)
-    ref = oracle_mod.gemm_i4(a_d.cpu().numpy(), b_d[n - 50:].cpu().numpy())
-    assert oracle_mod.compare(np.ascontiguousarray(c_d[:, n - 50:].cpu().numpy()), ref) == -1
+    block = ((2 ** 31 - 2) // kb) & ~255
+    assert 0 < block < n
+    for m in (8, 300):
+        a_d = torch.randint(-128, 128, (m, kb), dtype=torch.int8, device=DEV, generator=g)
+        assert qm.workspace_bytes(m, n, k) == 0
+        c_d = poisoned_c(m, n, DEV)
+        quadmul.gemm(a_d, b_d, c_d, m, n, k)
+        torch.cuda.synchronize()
+        for c0 in range(0, n, 262144):
+            cols = min(262144, n - c0)
+            part = torch.empty((m, cols), dtype=torch.int32, device=DEV)
+            qm.gemm(a_d, b_d[c0:c0 + cols], part, m, cols, k)
+            assert torch.equal(c_d[:, c0:c0 + cols], part), (m, c0)
+        for c0 in (0, block - 30, n - 50):
+            ref = oracle_mod.gemm_i4(a_d.cpu().numpy(), b_d[c0:c0 + 50].cpu().numpy())
+            assert oracle_mod.compare(np.ascontiguousarray(c_d[:, c0:c0 + 50].cpu().numpy()), ref) == -1
+        # the scaled output: column scales follow the blocks
+        rs = torch.rand(m, device=DEV, generator=g) * 0.01 + 0.001
+        cs = torch.rand(n, device=DEV, generator=g) + 0.5
+        d_d = torch.zeros((m, n), dtype=torch.bfloat16, device=DEV)
+        quadmul.gemm_scaled(a_d, b_d, d_d, m, n, k, rs, cs)
+        torch.cuda.synchronize()
+        for c0 in (0, block - 30, n - 50):
+            ref = oracle_mod.scale_round16(np.ascontiguousarray(c_d[:, c0:c0 + 50].cpu().numpy()), rs.cpu().numpy(), cs[c0:c0 + 50].cpu().numpy(),
+                                           oracle_mod.OUT_BF16)
+            assert np.array_equal(np.ascontiguousarray(d_d[:, c0:c0 + 50].view(torch.int16).cpu().numpy()).view(np.uint16), ref), (m, c0)
+        del a_d, c_d, d_d
 
 
 def test_host_threads_on_their_own_streams():
