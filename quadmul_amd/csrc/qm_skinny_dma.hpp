@@ -426,19 +426,46 @@ gemm_skinny_stream_dma_kernel(const GemmArgs p, const int nblocks)
                         __hip_atomic_fetch_add(&rh[((i * FN + j) * 4 + e) * 64 + lane], acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
         __syncthreads();
-        // One output element per thread and pass: element (m, n) of a block sits in register
-        // n % 4 of lane m + 16 (n / 4); 16 consecutive threads write 64 contiguous bytes of a row.
+        // Block bb is stored (and its sums cleared for the block after next) by wave bb % NW:
+        // lane (r, g) holds C[16 i + r][n0 + 16 j + 4 g .. + 3] in register order, four reads of
+        // 64 consecutive words each, 16 bytes per lane to C.
         const int n0 = blk * Cfg::BN;
-        for (int idx = tid; idx < FM * FN * 256; idx += Cfg::THREADS) {
-            const int bb = idx >> 8, ml = (idx >> 4) & 15, nl = idx & 15;
-            int32_t *const at_red = &rh[(bb * 4 + (nl & 3)) * 64 + ml + 16 * (nl >> 2)];
-            const int32_t s = *at_red;
-            *at_red = 0;
-            const int m = (bb / FN) * 16 + ml, n = n0 + (bb % FN) * 16 + nl;
-            if (m < p.M && n < p.N) {
-                const size_t at = (size_t)m * c_stride(p) + n;
-                if (p.out == OUT_I32) p.C[at] = s >> 8;
-                else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s >> 8, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);
+        const bool vec_ok = (c_stride(p) & 3) == 0 && ((uintptr_t)p.C & (p.out == OUT_I32 ? 15 : 7)) == 0;
+        for (int bb = wave; bb < FM * FN; bb += NW) {
+            v4i s;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                int32_t *const at_red = &rh[(bb * 4 + e) * 64 + lane];
+                s[e] = *at_red >> 8;
+                *at_red = 0;
+            }
+            const int m = (bb / FN) * 16 + r, n = n0 + (bb % FN) * 16 + 4 * g;
+            if (m >= p.M || n >= p.N) continue;
+            const size_t at = (size_t)m * c_stride(p) + n;
+            if (p.out == OUT_I32) {
+                if (vec_ok) {
+                    *reinterpret_cast<v4i *>(p.C + at) = s;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < p.N) p.C[at + e] = s[e];
+                }
+            } else {
+                uint16_t *const d = reinterpret_cast<uint16_t *>(p.C) + at;
+                const float rs = scale_at(p.row_scale, m, p.M);
+                uint16_t h[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int c = s[e];
+                    h[e] = round16(scaled(c, rs, scale_at(p.col_scale, n + e, p.N)), p.out);
+                }
+                if (vec_ok) {
+                    *reinterpret_cast<v2i *>(d) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < p.N) d[e] = h[e];
+                }
             }
         }
     }
