@@ -158,7 +158,7 @@ def test_selection_rules():
     # LDS, with a persistent grid and A resident in registers ("p") while the waves hold all of
     # K, the plain form ("d") beyond
     assert name(16, 4096, 4096) == "p1x1_w8_r2k2" and name(64, 4096, 4096) == "d4x1_w8_r1"
-    assert name(1, 4096, 4096) == "v1x1_w8_u4" and name(2, 5120, 5120) == "v2x1_w16_u2"   # dot-product kernel
+    assert name(1, 4096, 4096) == "v1x1_w4_u8" and name(1, 11008, 2048) == "v1x1_w8_u4" and name(2, 5120, 5120) == "v2x1_w16_u2"   # dot-product kernel
     assert name(1, 4096, 8192) == "v1x1_w16_u2" and name(2, 4096, 4096) == "v2x1_w8_u4"
     assert name(9, 28672, 14336) == "d1x1_w16_r1" and name(9, 11008, 8192) == "p1x1_w16_r2k2" and name(12, 2048, 2048) == "d1x1_w16_r1"
     assert name(3, 28672, 2048) == "p1x1_w8_r2k2" and name(16, 4096, 8192) == "d1x1_w16_r1"
