@@ -714,3 +714,39 @@ def test_skinny_kernels_streaming_global_to_lds(oracle_mod, shape):
     assert "d" in ran and (k > 8192 or m > 32 or "p" in ran), ran
     if m > 2:
         assert qm.config_name(qm.select_config(m, n, k) & 0xFFFF)[0] in "dp"
+
+
+def test_every_config_on_random_shapes_against_the_generic_kernel():
+    """A bounded soak: every configuration on random shapes it supports, ragged in all three
+    dimensions, with and without a K split, against the generic kernel on the same operands
+    (one thread per element, itself checked against the oracle above)."""
+    rng = np.random.default_rng(SEED_BASE + 77)
+    names = qm.config_names()
+    generic = names.index("generic")
+    skinny_m = [1, 2, 3, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64]
+    skinny_n = [1, 5, 16, 17, 100, 255, 256, 1000, 4096, 4100, 9000]
+    skinny_k = [1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 32, 33, 64, 100, 127, 128, 129, 256, 300]
+    tile_m = [1, 16, 63, 64, 65, 128, 200, 256, 257, 512, 700]
+    tile_n = [8, 64, 100, 128, 256, 260, 512, 1000, 1300]
+    tile_k = [1, 2, 3, 4, 5, 8, 12, 13, 16, 31, 32, 40, 64, 65]
+    ran = {}
+    for _ in range(20000):
+        cfg = int(rng.integers(len(names)))
+        if cfg == generic:
+            continue
+        tile = names[cfg][0] == "q"
+        m = int(rng.choice(tile_m if tile else skinny_m))
+        n = int(rng.choice(tile_n if tile else skinny_n))
+        k = 32 * int(rng.choice(tile_k if tile else skinny_k))
+        if not qm.config_supports(cfg, m, n, k):
+            continue
+        a = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=DEV)
+        b = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=DEV)
+        want = poisoned_c(m, n, DEV)
+        qm.gemm_cfg(a, b, want, m, n, k, generic)
+        ksplit = int(rng.choice([1, 1, 2, 3])) if tile and k >= 256 else 1
+        got = poisoned_c(m, n, DEV)
+        qm.gemm_cfg(a, b, got, m, n, k, cfg | (ksplit << 24) if ksplit > 1 else cfg, workspace=True if rng.integers(2) else None)
+        assert torch.equal(want, got), (names[cfg], ksplit, m, n, k)
+        ran[names[cfg]] = ran.get(names[cfg], 0) + 1
+    assert len(ran) == len(names) - 1 and min(ran.values()) >= 10, ran
