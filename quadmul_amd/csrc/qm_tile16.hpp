@@ -133,7 +133,14 @@ struct Tile16Cfg {
     // fits beside the ring of every co-resident workgroup.
     static constexpr int XPOSE_PITCH = 64 * 4 + 16, XPOSE_BYTES = 16 * XPOSE_PITCH;
     static constexpr bool XPOSE = FN % 4 == 0 && OCC * (RING_BYTES + WAVES * XPOSE_BYTES) <= 160 * 1024;
-    static constexpr int LDS_BYTES = RING_BYTES + (XPOSE ? WAVES * XPOSE_BYTES : 0);
+    // Where that does not fit: half the area, 16 rows x 32 int32 without padding -- the 16-byte
+    // chunk c of row r sits at chunk c ^ ((r >> 1) & 7), which keeps the 16 lanes of a write
+    // (one row each) and of a read (two rows of eight chunks) in different banks.
+    // (Measured on the tiles built for two workgroups per CU: 2-4 % on 256x128, nothing to
+    // -1.5 % on the 64- and 128-row tiles, whose blocks keep going out as they are.)
+    static constexpr int XHALF_BYTES = 16 * 128;
+    static constexpr bool XHALF = !XPOSE && FN % 2 == 0 && BM * BN >= 256 * 128 && OCC * (RING_BYTES + WAVES * XHALF_BYTES) <= 160 * 1024;
+    static constexpr int LDS_BYTES = RING_BYTES + (XPOSE ? WAVES * XPOSE_BYTES : XHALF ? WAVES * XHALF_BYTES : 0);
     // one DMA piece = one wave-wide 16-byte-per-lane load = 16 rows x 64 bytes
     static constexpr int A_PIECES = BM / 16 / WAVES, B_PIECES = BN / 16 / WAVES;
     static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile is a multiple of 16x16");
@@ -472,6 +479,46 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         if constexpr (t == 6) { read_back(std::integral_constant<int, 3>{}); store_rows(std::integral_constant<int, 1>{}); }
         if constexpr (t == 7) { store_rows(std::integral_constant<int, 2>{}); store_rows(std::integral_constant<int, 3>{}); }
     };
+    // Whole tile through the half-size area: part t = 0..3 of blocks (ib, 2*h) and (ib, 2*h + 1).
+    // Parts 0 and 1 write a block each -- and store the two row octets (8 rows x 128 bytes, eight
+    // consecutive lanes per row) that the half group before this one read back in its parts 2
+    // and 3; the last half group of a tile leaves its two for flush_half().
+    const uint32_t lane_half = ((uint32_t)(wm * Cfg::WM + (lane >> 3)) * (uint32_t)ldc + (uint32_t)(wn * Cfg::WN + (lane & 7) * 4)) * (uint32_t)ESZ;
+    uint8_t *const xh = smem + Cfg::RING_BYTES + wave * Cfg::XHALF_BYTES;
+    const int xh_wr = r * 128 + ((g ^ ((r >> 1) & 7)) << 4);                      // block 2h; block 2h + 1 is 64 bytes (chunk bit 2) away
+    const int xh_rd = (lane >> 3) * 128 + (((lane & 7) ^ (lane >> 4)) << 4);      // rows 0..7; rows 8..15: + 1024, chunk bit 2 flipped
+    auto store_half = [&](auto ib_, auto h_, auto k_) __attribute__((always_inline)) {
+        constexpr int ib = decltype(ib_)::value, h = decltype(h_)::value, k = decltype(k_)::value;
+        char *const at = tile_c + ((size_t)(ib * 16 + 8 * k) * ldc + h * 32) * ESZ;  // wave-uniform
+        if constexpr (OUT == OUT_I32) {
+            v4i v = xr[k];
+            v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
+            *reinterpret_cast<v4i *>(at + lane_half) = v;
+        } else {
+            *reinterpret_cast<v2i *>(at + lane_half) = pack16(xr[k]);
+        }
+    };
+    auto write_half = [&](auto ib_, auto h_, auto t_) __attribute__((always_inline)) {
+        constexpr int ib = decltype(ib_)::value, h = decltype(h_)::value, t = decltype(t_)::value;
+        constexpr int pib = h > 0 ? ib : ib - 1, ph = h > 0 ? h - 1 : FN / 2 - 1;  // the half group before this one
+        if constexpr (t < 2) {
+            const int at = t == 0 ? xh_wr : xh_wr ^ 64;
+            if constexpr (OUT == OUT_I32) {
+                const uint32_t at_lds = lds0 + Cfg::RING_BYTES + wave * Cfg::XHALF_BYTES + at;
+                asm volatile("ds_write_b128 %0, %1" ::"v"(at_lds), "a"(acc[ib][2 * h + t]) : "memory");
+                mfma16_zero(acc[ib][2 * h + t], zero4);
+            } else {
+                *reinterpret_cast<v4i *>(xh + at) = take_block(ib_, std::integral_constant<int, 2 * h + t>{});
+            }
+            if constexpr (pib >= 0) store_half(std::integral_constant<int, pib>{}, std::integral_constant<int, ph>{}, t_);
+        }
+        if constexpr (t == 2) xr[0] = *reinterpret_cast<const v4i *>(xh + xh_rd);
+        if constexpr (t == 3) xr[1] = *reinterpret_cast<const v4i *>(xh + ((xh_rd + 1024) ^ 64));
+    };
+    auto flush_half = [&]() __attribute__((always_inline)) {
+        store_half(std::integral_constant<int, FM - 1>{}, std::integral_constant<int, FN / 2 - 1>{}, std::integral_constant<int, 0>{});
+        store_half(std::integral_constant<int, FM - 1>{}, std::integral_constant<int, FN / 2 - 1>{}, std::integral_constant<int, 1>{});
+    };
     // Whole tile, no room in the LDS: block (ib, j) stored as it is, in two parts.
     auto write_block = [&](auto ib_, auto j_, auto t_) __attribute__((always_inline)) {
         constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value, t = decltype(t_)::value;
@@ -487,6 +534,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     auto write_whole = [&](auto ib_, auto s_) __attribute__((always_inline)) {
         constexpr int s = decltype(s_)::value;
         if constexpr (Cfg::XPOSE) write_group(ib_, std::integral_constant<int, s / 8>{}, std::integral_constant<int, s % 8>{});
+        else if constexpr (Cfg::XHALF) write_half(ib_, std::integral_constant<int, s / 4>{}, std::integral_constant<int, s % 4>{});
         else write_block(ib_, std::integral_constant<int, s / 2>{}, std::integral_constant<int, s % 2>{});
     };
     // Any tile: guarded stores (ragged edges, odd N or unaligned C, K-split partial sums)
@@ -623,7 +671,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         // counter counts loads and stores alike, in order of issue: the stores of a last
         // step are all younger than the loads that must have landed, and are allowed to stay
         // in flight as well (the counter cannot express more than 63).
-        constexpr int pending = (AHEAD - 2) * NP + (last ? (FM - 1) * FN : 0);
+        // (through the half-size area the last two stores of row FM-2 go out with row FM-1, after this step)
+        constexpr int pending = (AHEAD - 2) * NP + (last ? (FM - 1) * FN - (Cfg::XHALF ? 2 : 0) : 0);
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(pending > 63 ? 63 : pending) : "memory");
         const int t = ring[0];
 #pragma unroll
@@ -699,6 +748,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 write_whole(std::integral_constant<int, FM - 1>{}, s_);
                 __builtin_amdgcn_sched_barrier(0);
             });
+            if constexpr (Cfg::XHALF) flush_half();
         } else {
             static_for<0, FM>([&](auto ib_) {
                 static_for<0, FN>([&](auto j_) {
