@@ -348,7 +348,7 @@ static int run_gemm(const void *A, const void *B, void *dst, int m, int n, int k
         PadPlan pl = plan_padded_k(m, n, k, align, ch);
         if (pl.on && !launcher(pl.ch.cfg)) {
             // a pipelined configuration that has the scaled output, if the shape is one for those
-            const int id = find_config("q256x256_w2x2_s4o1");
+            const int id = find_config("q256x256_w2x2_s9o1");
             if (id >= 0 && launcher(id)) pl.ch.cfg = id; else pl.on = false;
         }
         if (pl.on && ((uintptr_t)workspace & 15) == 0 && workspace_bytes >= pl.bytes()) {

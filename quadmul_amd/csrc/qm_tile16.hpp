@@ -126,7 +126,17 @@ struct Tile16Cfg {
     static constexpr int A_BYTES = BM * PITCH, B_BYTES = BN * PITCH;
     static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int STAGES = STAGES_;  // LDS ring depth: 4 or 5 on the large tiles; 6 to 8 on the small ones, whose K-steps are short against the latency of HBM
-    static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+    // STAGES = 9 is the paired ring: five stages of A and four of B, each operand in a ring of
+    // its own, filled two K-steps at a time.  A K-step takes 64 bytes of every row, half a
+    // 128-byte cache line; loading the halves of a line a K-step apart fetches the line twice
+    // (64 KiB of other lines pass through the 32 KiB L1 of the CU in between).  The paired ring
+    // issues the loads of steps 2n and 2n+1 of the same rows back to back, in every other
+    // step.  Both target stages must be free then and the data is needed one step before its
+    // MFMAs: A's stage frees when its step ends (5 stages), B's when its step begins (its
+    // fragments are read and widened a step ahead: 4 stages).
+    static constexpr bool PAIR = STAGES_ == 9;
+    static constexpr int A_STAGES = PAIR ? 5 : STAGES_, B_STAGES = PAIR ? 4 : STAGES_;
+    static constexpr int RING_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
     // Per-wave LDS area through which finished accumulator blocks are turned into row-major
     // order before they are stored: 16 rows x 64 int32, rows padded by 16 bytes so that the
     // 16 lanes of a ds_write_b128 (one row each) fall into different banks.  Used when it
@@ -134,8 +144,8 @@ struct Tile16Cfg {
     static constexpr int XPOSE_PITCH = 64 * 4 + 16, XPOSE_BYTES = 16 * XPOSE_PITCH;
     static constexpr bool XPOSE = FN % 4 == 0 && OCC * (RING_BYTES + WAVES * XPOSE_BYTES) <= 160 * 1024;
     // Where that does not fit: half the area, 16 rows x 32 int32 without padding -- the 16-byte
-    // chunk c of row r sits at chunk c ^ ((r >> 1) & 7), which keeps the 16 lanes of a write
-    // (one row each) and of a read (two rows of eight chunks) in different banks.
+    // chunk c of row r sits at chunk c ^ (r & 7), which keeps eight consecutive lanes of a
+    // write (one row each) and of a read (the eight chunks of a row) in different banks.
     // (Measured on the tiles built for two workgroups per CU: 2-4 % on 256x128, nothing to
     // -1.5 % on the 64- and 128-row tiles, whose blocks keep going out as they are.)
     static constexpr int XHALF_BYTES = 16 * 128;
@@ -146,7 +156,8 @@ struct Tile16Cfg {
     static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile is a multiple of 16x16");
     static_assert(BM % (16 * WAVES) == 0 && BN % (16 * WAVES) == 0, "DMA pieces must divide evenly among the waves");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
-    static_assert(STAGES >= 3 && STAGES <= 8, "ring depth");
+    static_assert(STAGES >= 3 && STAGES <= 9, "ring depth");
+    static_assert(!PAIR || A_PIECES + B_PIECES <= FM, "the paired ring issues at most one piece of each of its two steps per sub-step");
     static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
     static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
     static_assert((W_OPS * FN) % FM == 0, "B widening must split evenly over the sub-steps");
@@ -261,16 +272,23 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             b_goff[q] = (uint32_t)min((n0 + q * WAVES * 16) + dma_base, p.N - 1) * (uint32_t)Kb + dma_col;
     };
     const uint8_t *a_src, *b_src;  // operand base + K offset of the step the cursor points at
+    const uint8_t *a_src2 = nullptr, *b_src2 = nullptr;  // paired ring: the same for the step after it
     auto cursor_point = [&]() __attribute__((always_inline)) {
         const int step = d_kt0 + min(d_kt, d_KT - 1);
         const int kofs = (TAIL && k_tail != 0 && step == kt_all - 1) ? Kb - BK / 2 : step * (BK / 2);
         a_src = p.A + kofs;
         b_src = p.B + kofs;
+        if constexpr (Cfg::PAIR) {
+            const int step2 = d_kt0 + min(d_kt + 1, d_KT - 1);
+            const int kofs2 = (TAIL && k_tail != 0 && step2 == kt_all - 1) ? Kb - BK / 2 : step2 * (BK / 2);
+            a_src2 = p.A + kofs2;
+            b_src2 = p.B + kofs2;
+        }
     };
     // Past the last item the cursor stays on the last step: those loads land in stages
     // nobody reads any more.
     auto cursor_advance = [&]() __attribute__((always_inline)) {
-        ++d_kt;
+        d_kt += Cfg::PAIR ? 2 : 1;  // (an item's steps come in pairs: two steps on never pass the item's end)
         if (d_kt >= d_KT + (d_KT & 1)) {
             if (d_item + G < nitems) {
                 d_item += G;
@@ -311,11 +329,29 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         else asm volatile("global_load_lds_dwordx4 %0, %1" ::"v"(b_goff[piece - A_PIECES]), "s"(b_src) : "memory");
     };
 
+    // Paired ring: piece q of the cursor's step (second = false) or of the step after it, into
+    // the stage at byte offset `at` of that operand's ring.
+    auto pair_setup = [&](int piece, int at) __attribute__((always_inline)) {
+        const uint32_t dst = dma_lds + at + (piece < A_PIECES ? piece : piece - A_PIECES) * WAVES * 16 * PITCH;
+        asm volatile("s_mov_b32 m0, %0" ::"s"(dst) : "memory", "m0");
+    };
+    auto pair_issue = [&](int piece, bool second) __attribute__((always_inline)) {
+        if (piece < A_PIECES) asm volatile("global_load_lds_dwordx4 %0, %1" ::"v"(a_goff[piece]), "s"(second ? a_src2 : a_src) : "memory");
+        else asm volatile("global_load_lds_dwordx4 %0, %1" ::"v"(b_goff[piece - A_PIECES]), "s"(second ? b_src2 : b_src) : "memory");
+    };
+    auto pair_piece = [&](int piece, int at, bool second) __attribute__((always_inline)) {
+        const uint32_t dst = dma_lds + at + (piece < A_PIECES ? piece : piece - A_PIECES) * WAVES * 16 * PITCH;
+        if (piece < A_PIECES)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(a_goff[piece]), "s"(second ? a_src2 : a_src) : "memory", "m0");
+        else
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(b_goff[piece - A_PIECES]), "s"(second ? b_src2 : b_src) : "memory", "m0");
+    };
+
     // ---- fragment reads: lane -> row r of a 16-row fragment, chunk g (32 nibbles) ----
     // (rows of consecutive fragments differ by 16, which leaves (row >> 1) & 3 unchanged)
     const int a_row = wm * Cfg::WM + r, b_row = wn * Cfg::WN + r;
     const int a_rd = a_row * PITCH + ((g ^ ((a_row >> 1) & 3)) << 4);
-    const int b_rd = Cfg::A_BYTES + b_row * PITCH + ((g ^ ((b_row >> 1) & 3)) << 4);
+    const int b_rd = (Cfg::PAIR ? 0 : Cfg::A_BYTES) + b_row * PITCH + ((g ^ ((b_row >> 1) & 3)) << 4);  // (paired ring: the B stages have offsets of their own)
     auto read_a = [&](int stage_byte, int i) -> v4i {
         return *reinterpret_cast<const v4i *>(smem + stage_byte + a_rd + i * 16 * PITCH);
     };
@@ -333,16 +369,30 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
 
     // ---- prologue: steps 0 .. STAGES-2 of the stream on their way into stages 0 .. STAGES-2;
     // wait for 0 and 1 ----
-    constexpr int STAGES = Cfg::STAGES, AHEAD = STAGES - 1;  // step s+AHEAD is issued during step s
+    constexpr int STAGES = Cfg::PAIR ? 4 : Cfg::STAGES, AHEAD = STAGES - 1;  // step s+AHEAD is issued during step s (paired ring: steps s+3 and s+4 during every odd step s)
+    constexpr int B_BASE = Cfg::A_STAGES * Cfg::A_BYTES;  // paired ring: where the B stages begin
     cursor_load();
     cursor_point();
+    if constexpr (Cfg::PAIR) {
+        // steps 0..3 into stages 0..3 of both rings; wait for 0 and 1
 #pragma unroll
-    for (int t = 0; t < AHEAD; ++t) {
+        for (int t = 0; t < 4; t += 2) {
 #pragma unroll
-        for (int q = 0; q < NP; ++q) dma_piece(q, t * STAGE);
-        cursor_advance();
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int q = 0; q < NP; ++q) pair_piece(q, q < A_PIECES ? (t + h) * Cfg::A_BYTES : B_BASE + (t + h) * Cfg::B_BYTES, h == 1);
+            cursor_advance();
+        }
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NP) : "memory");
+    } else {
+#pragma unroll
+        for (int t = 0; t < AHEAD; ++t) {
+#pragma unroll
+            for (int q = 0; q < NP; ++q) dma_piece(q, t * STAGE);
+            cursor_advance();
+        }
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 2) * NP) : "memory");
     }
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((AHEAD - 2) * NP) : "memory");
     __syncthreads();
 
     // B fragments of the current step (widened) and of the next (being widened); the two
@@ -351,7 +401,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     v4i b_ev[2][FN], b_od[2][FN], b_pk[2];
     v4i a_ev[2], a_od[2], a_pk[2];
 #pragma unroll
-    for (int j = 0; j < FN; ++j) x16_expand(read_b(0, j), b_ev[0][j], b_od[0][j]);
+    for (int j = 0; j < FN; ++j) x16_expand(read_b(Cfg::PAIR ? B_BASE : 0, j), b_ev[0][j], b_od[0][j]);
     x16_expand(read_a(0, 0), a_ev[0], a_od[0]);
     a_pk[1] = read_a(0, 1);
 
@@ -359,6 +409,16 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     int ring[STAGES];
 #pragma unroll
     for (int t = 0; t < STAGES; ++t) ring[t] = t * STAGE;
+    // Paired ring, during step s: a_ring[t] holds (or waits for) A of step s+t, t = 0..4;
+    // b_ring[t] B of step s+t, t = 1..3, and b_ring[0] is free (B of step s went into
+    // registers during step s-1).
+    int a_ring[Cfg::PAIR ? 5 : 1], b_ring[Cfg::PAIR ? 4 : 1];
+    if constexpr (Cfg::PAIR) {
+#pragma unroll
+        for (int t = 0; t < 5; ++t) a_ring[t] = t * Cfg::A_BYTES;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) b_ring[t] = B_BASE + t * Cfg::B_BYTES;
+    }
 
     // Widening op k (0..W-1) of a packed fragment, W = 10: for each half (dwords 2h, 2h+1) one
     // 64-bit shift of the pair (the nibble that crosses into the upper dword is masked away
@@ -485,8 +545,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // and 3; the last half group of a tile leaves its two for flush_half().
     const uint32_t lane_half = ((uint32_t)(wm * Cfg::WM + (lane >> 3)) * (uint32_t)ldc + (uint32_t)(wn * Cfg::WN + (lane & 7) * 4)) * (uint32_t)ESZ;
     uint8_t *const xh = smem + Cfg::RING_BYTES + wave * Cfg::XHALF_BYTES;
-    const int xh_wr = r * 128 + ((g ^ ((r >> 1) & 7)) << 4);                      // block 2h; block 2h + 1 is 64 bytes (chunk bit 2) away
-    const int xh_rd = (lane >> 3) * 128 + (((lane & 7) ^ (lane >> 4)) << 4);      // rows 0..7; rows 8..15: + 1024, chunk bit 2 flipped
+    const int xh_wr = r * 128 + ((g ^ (r & 7)) << 4);                             // block 2h; block 2h + 1 is 64 bytes (chunk bit 2) away
+    const int xh_rd = (lane >> 3) * 128 + (((lane & 7) ^ (lane >> 3)) << 4);      // rows 0..7; rows 8..15: + 1024
     auto store_half = [&](auto ib_, auto h_, auto k_) __attribute__((always_inline)) {
         constexpr int ib = decltype(ib_)::value, h = decltype(h_)::value, k = decltype(k_)::value;
         char *const at = tile_c + ((size_t)(ib * 16 + 8 * k) * ldc + h * 32) * ESZ;  // wave-uniform
@@ -513,7 +573,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             if constexpr (pib >= 0) store_half(std::integral_constant<int, pib>{}, std::integral_constant<int, ph>{}, t_);
         }
         if constexpr (t == 2) xr[0] = *reinterpret_cast<const v4i *>(xh + xh_rd);
-        if constexpr (t == 3) xr[1] = *reinterpret_cast<const v4i *>(xh + ((xh_rd + 1024) ^ 64));
+        if constexpr (t == 3) xr[1] = *reinterpret_cast<const v4i *>(xh + xh_rd + 1024);
     };
     auto flush_half = [&]() __attribute__((always_inline)) {
         store_half(std::integral_constant<int, FM - 1>{}, std::integral_constant<int, FN / 2 - 1>{}, std::integral_constant<int, 0>{});
@@ -609,10 +669,11 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     //    sub-step, and the A fragment two sub-steps ahead --
                     static_for<0, FN>([&](auto j_) {
                         constexpr int j = decltype(j_)::value;
-                        if constexpr ((W * j) / BSHARE == i) b_pk[j & 1] = read_b(ring[1], j);
+                        if constexpr ((W * j) / BSHARE == i) b_pk[j & 1] = read_b(Cfg::PAIR ? b_ring[1] : ring[1], j);
                     });
                     constexpr int i2 = i + 2;
-                    a_pk[pa] = read_a(i2 >= FM ? ring[1] : ring[0], i2 % FM);
+                    if constexpr (Cfg::PAIR) a_pk[pa] = read_a(i2 >= FM ? a_ring[1] : a_ring[0], i2 % FM);
+                    else a_pk[pa] = read_a(i2 >= FM ? ring[1] : ring[0], i2 % FM);
                 } else {
                     // -- this slot's share of the widening work: ops [lo, hi) of the sub-step's
                     //    list: W ops for the next A fragment, then BSHARE ops of the next B --
@@ -634,15 +695,29 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 // (With a ring of three stages the loads issued in a step must have landed
                 // at its end.  In a last step they all go out in sub-step 0, ahead of the
                 // first store, so that "all but the stores" can be waited for.)
-                constexpr bool bunched = last && AHEAD == 2;
-                constexpr bool split = !bunched && NP <= FM && SLOTS >= 4;  // at most one piece per sub-step
+                constexpr bool bunched = !Cfg::PAIR && last && AHEAD == 2;
+                constexpr bool split = !Cfg::PAIR && !bunched && NP <= FM && SLOTS >= 4;  // at most one piece per sub-step
+                if constexpr (Cfg::PAIR && bs == 1) {
+                    // paired ring, odd steps: piece i of step s+3 in the first half of the sub-step,
+                    // the same rows of step s+4 (the other half of their cache lines) in the second
+                    static_assert(!Cfg::PAIR || SLOTS >= 8, "two loads per sub-step, each with its M0 two slots ahead");
+                    static_for<0, NP>([&](auto q_) {
+                        constexpr int q = decltype(q_)::value;
+                        if constexpr (q * FM / NP == i) {
+                            if constexpr (s == SLOTS / 2 - 3) pair_setup(q, q < A_PIECES ? a_ring[3] : b_ring[3]);
+                            if constexpr (s == SLOTS / 2 - 1) pair_issue(q, false);
+                            if constexpr (s == SLOTS - 3) pair_setup(q, q < A_PIECES ? a_ring[4] : b_ring[0]);
+                            if constexpr (s == SLOTS - 1) pair_issue(q, true);
+                        }
+                    });
+                }
                 if constexpr (split && s == SLOTS - 3) {
                     static_for<0, NP>([&](auto q_) {
                         constexpr int q = decltype(q_)::value;
                         if constexpr (q * FM / NP == i) dma_setup(q, ring[STAGES - 1]);
                     });
                 }
-                if constexpr (s == SLOTS - 1) {
+                if constexpr (!Cfg::PAIR && s == SLOTS - 1) {
                     static_for<0, NP>([&](auto q_) {
                         constexpr int q = decltype(q_)::value;
                         if constexpr (split) {
@@ -672,13 +747,27 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         // step are all younger than the loads that must have landed, and are allowed to stay
         // in flight as well (the counter cannot express more than 63).
         // (through the half-size area the last two stores of row FM-2 go out with row FM-1, after this step)
-        constexpr int pending = (AHEAD - 2) * NP + (last ? (FM - 1) * FN - (Cfg::XHALF ? 2 : 0) : 0);
+        // (paired ring: an odd step has issued the loads of two steps, all younger than what must
+        // have landed; after an even step, which issues none, the youngest load belongs to step
+        // s+3 and the one before it to s+2, which must be there)
+        constexpr int pending = (Cfg::PAIR ? (bs == 1 ? 2 * NP : 1) : (AHEAD - 2) * NP) + (last ? (FM - 1) * FN - (Cfg::XHALF ? 2 : 0) : 0);
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(pending > 63 ? 63 : pending) : "memory");
-        const int t = ring[0];
+        if constexpr (Cfg::PAIR) {
+            const int ta = a_ring[0], tb = b_ring[0];
 #pragma unroll
-        for (int u = 0; u + 1 < STAGES; ++u) ring[u] = ring[u + 1];
-        ring[STAGES - 1] = t;
-        cursor_advance();
+            for (int u = 0; u < 4; ++u) a_ring[u] = a_ring[u + 1];
+            a_ring[4] = ta;
+#pragma unroll
+            for (int u = 0; u < 3; ++u) b_ring[u] = b_ring[u + 1];
+            b_ring[3] = tb;
+            if constexpr (bs == 1) cursor_advance();
+        } else {
+            const int t = ring[0];
+#pragma unroll
+            for (int u = 0; u + 1 < STAGES; ++u) ring[u] = ring[u + 1];
+            ring[STAGES - 1] = t;
+            cursor_advance();
+        }
     };
 
     // One item: K-steps in pairs; when the item has an odd number of them, the second of the
