@@ -157,7 +157,6 @@ struct Tile16Cfg {
     static_assert(BM % (16 * WAVES) == 0 && BN % (16 * WAVES) == 0, "DMA pieces must divide evenly among the waves");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
     static_assert(STAGES >= 3 && STAGES <= 9, "ring depth");
-    static_assert(!PAIR || A_PIECES + B_PIECES <= FM, "the paired ring issues at most one piece of each of its two steps per sub-step");
     static_assert(OCC * LDS_BYTES <= 160 * 1024, "co-resident workgroups must fit the LDS together");
     static_assert(FM >= 2 && FM % 2 == 0 && FN >= 1, "pipeline needs an even number (>= 2) of A fragments per wave");
     static_assert((W_OPS * FN) % FM == 0, "B widening must split evenly over the sub-steps");
@@ -700,14 +699,18 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 if constexpr (Cfg::PAIR && bs == 1) {
                     // paired ring, odd steps: piece i of step s+3 in the first half of the sub-step,
                     // the same rows of step s+4 (the other half of their cache lines) in the second
-                    static_assert(!Cfg::PAIR || SLOTS >= 8, "two loads per sub-step, each with its M0 two slots ahead");
                     static_for<0, NP>([&](auto q_) {
                         constexpr int q = decltype(q_)::value;
                         if constexpr (q * FM / NP == i) {
-                            if constexpr (s == SLOTS / 2 - 3) pair_setup(q, q < A_PIECES ? a_ring[3] : b_ring[3]);
-                            if constexpr (s == SLOTS / 2 - 1) pair_issue(q, false);
-                            if constexpr (s == SLOTS - 3) pair_setup(q, q < A_PIECES ? a_ring[4] : b_ring[0]);
-                            if constexpr (s == SLOTS - 1) pair_issue(q, true);
+                            // the pieces of this sub-step are q = first .. first + cnt - 1; each gets two loads,
+                            // `spacing` slots apart, M0 written two slots ahead of each
+                            constexpr int first = (i * NP + FM - 1) / FM, last1 = ((i + 1) * NP + FM - 1) / FM, cnt = last1 > first ? last1 - first : 1;
+                            constexpr int spacing = SLOTS / (2 * cnt), at1 = 2 * (q - first) * spacing + spacing - 1, at2 = at1 + spacing;
+                            static_assert(spacing >= 4, "too many pieces per sub-step for the slots it has");
+                            if constexpr (s == at1 - 2) pair_setup(q, q < A_PIECES ? a_ring[3] : b_ring[3]);
+                            if constexpr (s == at1) pair_issue(q, false);
+                            if constexpr (s == at2 - 2) pair_setup(q, q < A_PIECES ? a_ring[4] : b_ring[0]);
+                            if constexpr (s == at2) pair_issue(q, true);
                         }
                     });
                 }
