@@ -130,6 +130,7 @@ def time_graph(fn, launches=200, replays=5):
 # each scaled by what the same counter reads for a 256 MiB device-to-device copy); the
 # summaries are under profiles/.  Not measured in this run.
 PROFILED_TRAFFIC = {(8192, 8192, 8192): 673454571, (8000, 8000, 8064): 768061246, (4096, 4096, 4096): 118719686, (2048, 11008, 4096): 192246061,
+                    (2048, 4096, 11008): 124369042, (16, 28672, 4096): 60893081,
                     (1024, 1024, 1024): 7542887, (16, 4096, 4096): 8993197, (64, 4096, 4096): 10607970, (1, 4096, 4096): 8460539}
 PROFILED_TRAFFIC_OTHER = {"scaled_fp16_4096^3": 85807335, "quantize_pack_fp16_4096x4096": 42113123}
 
