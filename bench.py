@@ -7,10 +7,12 @@ A step is one call of ``quadmul.gemm`` (the drop-in entry point) on operands alr
 resident in HBM.  Prints ONE JSON line:
 
 * ``metric``/``value``/``roofline``: the headline workload, by default the largest
-  single-GPU configuration of the contract (M=N=K=8192): W untimed calls, then exactly K
-  calls between two ``torch.cuda.synchronize()`` (wall clock -> ``value``, ``ms_per_step``)
-  and, inside them, between two HIP events recorded on the stream the kernels are
-  launched on (average launch duration -> ``roofline.achieved``);
+  single-GPU configuration of the contract (M=N=K=8192): every input is made first, the
+  kernel runs untimed for ``--preheat-ms`` (``config.preheat_ms``: the power management
+  settles on the kernel's own load), then W untimed calls, then exactly K calls between
+  two ``torch.cuda.synchronize()`` (wall clock -> ``value``, ``ms_per_step``) with one HIP
+  event per step recorded on the stream the kernels are launched on (first to last:
+  average launch duration -> ``roofline.achieved``; median, min and max beside it);
 * ``targets``: every other configuration of the contract (1024^3, 4096^3, M in {1, 16, 64}
   at N=K=4096, the three M=2048 MLP shapes, 8000x8000x8064), each with its own
   ``roofline``.  These are timed the way the reference's harness times its kernel
@@ -27,8 +29,10 @@ resident in HBM.  Prints ONE JSON line:
 from __future__ import annotations
 
 import argparse
+import glob
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -79,22 +83,48 @@ def make_packed(m, n, k, seed):
     return pack(a), pack(b)
 
 
-def time_steps(fn, steps, warmup):
-    """(wall ms per step, event ms per step) over exactly `steps` calls."""
+def time_steps(fn, steps, warmup, preheat_ms=0.0):
+    """Exactly `steps` calls after `warmup` untimed ones: wall ms per step, and from one HIP
+    event per step on the launch stream the mean / median / min / max step in ms.
+
+    `preheat_ms` > 0: before the warm-ups the same kernel runs back to back for at least that
+    long, untimed.  A burst of launches that follows an idle GPU starts with a power-management
+    transient (the first four launches of 8192^3 at 0.36 ms, launches 6..12 at 0.43-0.46 ms,
+    then a slow return to the sustained 0.33 ms over about 80 launches = 30 ms, whatever the
+    length of the idle gap); the timing method this follows (kernel.cu:472-497: 10 warm-ups,
+    100 trials) averages over it, a run of 5 + 20 launches does not."""
     import torch
 
+    pre = {"preheat_ms": 0.0, "preheat_launches": 0}
+    if preheat_ms > 0:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        n = max(1, int(preheat_ms / max(e0.elapsed_time(e1), 1e-3)) + 1)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        pre_events = (e0, e1, n)
     for _ in range(warmup):
         fn()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
+    evs[0].record()
+    for i in range(steps):
         fn()
-    e1.record()
+        evs[i + 1].record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    return wall, e0.elapsed_time(e1) / steps
+    per = [evs[i].elapsed_time(evs[i + 1]) for i in range(steps)]
+    if preheat_ms > 0:
+        pre = {"preheat_ms": round(pre_events[0].elapsed_time(pre_events[1]), 1), "preheat_launches": pre_events[2]}
+    stats = {"mean": evs[0].elapsed_time(evs[steps]) / steps, "median": statistics.median(per), "min": min(per), "max": max(per)}
+    return wall, stats, pre
 
 
 def time_graph(fn, launches=200, replays=5):
@@ -125,32 +155,65 @@ def time_graph(fn, launches=200, replays=5):
     return statistics.median(ts), min(ts), max(ts)
 
 
-# Bytes moved per launch past the L2s, profiled offline: two rocprofv3 --pmc runs of
-# `bench.py --workload W --launches-only 20` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch,
-# each scaled by what the same counter reads for a 256 MiB device-to-device copy); the
-# summaries are under profiles/.  Not measured in this run.
-PROFILED_TRAFFIC = {(8192, 8192, 8192): 673454571, (8000, 8000, 8064): 768061246, (4096, 4096, 4096): 118719686, (2048, 11008, 4096): 192246061,
-                    (2048, 4096, 11008): 124369042, (16, 28672, 4096): 60893081,
-                    (1024, 1024, 1024): 7542887, (16, 4096, 4096): 8993197, (64, 4096, 4096): 10607970, (1, 4096, 4096): 8460539}
-PROFILED_TRAFFIC_OTHER = {"scaled_fp16_4096^3": 85807335, "quantize_pack_fp16_4096x4096": 42113123}
+# Bytes moved per launch past the L2s come from the committed rocprofv3 summaries, not from
+# this run: two --pmc runs of `bench.py --workload W --launches-only 20` (FETCH_SIZE, then
+# WRITE_SIZE; KiB per dispatch, each scaled by what the same counter reads for a 256 MiB
+# device-to-device copy) per workload, summarised in profiles/<kernel>_<configuration>__<W>.md.
+# A summary is used only while the configuration it profiled is still the one the library
+# chooses for that shape; a retuned table row leaves `traffic` null until it is profiled again.
+_TITLE = re.compile(r"^# (\S+?)_kernel, configuration (\S+?),(?: [^\n]*?)? on (\S+) \(M=(\d+) N=(\d+) K=(\d+)\)")
+_TOTAL = re.compile(r"^\| total \| \| (\d+) \|", re.M)
 
 
-def roofline_of(m, n, k, bound, ms, issue_peak_tops=None):
+def profile_summaries(root=None):
+    """{workload: {"path", "kernel", "config", "shape", "traffic"}} for every profiles/*__<workload>.md
+    with a traffic table."""
+    out = {}
+    for path in sorted(glob.glob(os.path.join(root or ROOT, "profiles", "*__*.md"))):
+        with open(path) as f:
+            text = f.read()
+        title = _TITLE.match(text)
+        total = _TOTAL.search(text)
+        if not title or not total:
+            continue
+        out[title.group(3)] = {"path": "profiles/" + os.path.basename(path), "kernel": title.group(1), "config": title.group(2),
+                               "shape": tuple(int(title.group(i)) for i in (4, 5, 6)), "traffic": int(total.group(1))}
+    return out
+
+
+def profile_total(workload):
+    """The traffic total of profiles/*__<workload>.md whatever its title says (summaries of the
+    kernels either side of the GEMM), or None."""
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", f"*__{workload}.md"))):
+        with open(path) as f:
+            total = _TOTAL.search(f.read())
+        if total:
+            return int(total.group(1))
+    return None
+
+
+def profiled_traffic(name, m, n, k, config):
+    """(bytes per launch, where from) for workload `name` running configuration `config`."""
+    prof = profile_summaries().get(name)
+    if prof is None:
+        return None, "no rocprofv3 summary of this workload under profiles/"
+    if prof["shape"] != (m, n, k) or prof["config"] != config:
+        return None, f"{prof['path']} profiled {prof['config']}, the library now chooses {config}: not used"
+    return prof["traffic"], f"rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiled offline ({prof['path']})"
+
+
+def roofline_of(m, n, k, bound, ms, issue_peak_tops=None, name=None, config=None):
     ops = 2.0 * m * n * k
+    traffic, source = profiled_traffic(name, m, n, k, config) if name else (None, None)
     if bound == "mfma":
-        achieved = ops / ms / 1e9  # TOP/s
-        r = {"bound": "mfma", "achieved": round(achieved, 1), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-             "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": PROFILED_TRAFFIC.get((m, n, k)),
-             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiled offline (profiles/)" if (m, n, k) in PROFILED_TRAFFIC else None,
-             "algorithmic_bytes": algorithmic_bytes(m, n, k), "launch_us": round(ms * 1e3, 3)}
-        if issue_peak_tops:
-            r["frac_of_measured_issue_peak"] = round(achieved / issue_peak_tops, 4)
-        return r
-    achieved = algorithmic_bytes(m, n, k) / ms / 1e6  # GB/s
-    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": PROFILED_TRAFFIC.get((m, n, k)),
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiled offline (profiles/)" if (m, n, k) in PROFILED_TRAFFIC else None,
-            "algorithmic_bytes": algorithmic_bytes(m, n, k), "launch_us": round(ms * 1e3, 3)}
+        achieved, peak, unit = ops / ms / 1e9, INT8_PEAK_TOPS, "TOP/s"
+    else:
+        achieved, peak, unit = algorithmic_bytes(m, n, k) / ms / 1e6, HBM_PEAK_GBS, "GB/s"
+    r = {"bound": bound, "achieved": round(achieved, 1), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4),
+         "traffic": traffic, "traffic_source": source, "algorithmic_bytes": algorithmic_bytes(m, n, k), "launch_us": round(ms * 1e3, 3)}
+    if bound == "mfma" and issue_peak_tops:
+        r["frac_of_measured_issue_peak"] = round(achieved / issue_peak_tops, 4)
+    return r
 
 
 def check_rows(ap, bp, c_d, m, count=8):
@@ -194,9 +257,10 @@ def run_target(name, issue_peak_tops):
     est_ms = max((time.perf_counter() - t0) * 1e3 * 0.5, 2e-3)
     launches = int(min(2000, max(20, 50.0 / est_ms)))
     med, lo, hi = time_graph(fn, launches=launches)
+    config = qm.config_name(qm.select_config(m, n, k) & 0xFFFF)
     out = {
         "workload": workload_text(name), "m": m, "n": n, "k": k,
-        "kernel": qm.config_name(qm.select_config(m, n, k) & 0xFFFF),
+        "kernel": config,
         "timing": f"HIP graph of {launches} launches, median of 5 replays",
         "ms_per_launch": round(med, 5), "ms_per_launch_min_max": [round(lo, 5), round(hi, 5)],
         "tops": round(2.0 * m * n * k / med / 1e9, 2),
@@ -207,28 +271,19 @@ def run_target(name, issue_peak_tops):
         # Launched again and again on the same B, the kernel reads B out of the L2s and the
         # 256 MiB memory-side cache, not HBM.  For the HBM roofline the launches of the graph
         # rotate over enough copies of B (each with a C of its own) to exceed that cache.
-        ncopies = max(2, -(-(320 << 20) // max(1, bp.numel())))
-        bs = [b_d] + [b_d.clone() for _ in range(ncopies - 1)]
-        cs = [c_d] + [torch.empty_like(c_d) for _ in range(ncopies - 1)]
-        turn = [0]
-
-        def fn_rot():
-            i = turn[0] % ncopies
-            turn[0] += 1
-            quadmul.gemm(a_d, bs[i], cs[i], m, n, k)
-
+        fn_rot, ncopies, cs = rotating_call(a_d, b_d, c_d, m, n, k)
         rot, rlo, rhi = time_graph(fn_rot, launches=5 * ncopies)
         for c_i in cs[1:]:
             assert torch.equal(c_i, c_d)
-        del bs, cs
+        del fn_rot, cs
         out["ms_per_launch_rotating_b"] = round(rot, 5)
         out["ms_per_launch_rotating_b_min_max"] = [round(rlo, 5), round(rhi, 5)]
-        out["roofline"] = roofline_of(m, n, k, bound, rot)
+        out["roofline"] = roofline_of(m, n, k, bound, rot, name=name + "_rotating_b", config=config)
         out["roofline"]["note"] = (f"launches rotate over {ncopies} copies of B (> 256 MiB memory-side cache): B comes from HBM; "
                                    f"graph of {5 * ncopies} launches, median of 5 replays")
-        out["roofline_b_cache_resident"] = roofline_of(m, n, k, bound, med)
+        out["roofline_b_cache_resident"] = roofline_of(m, n, k, bound, med, name=name, config=config)
     else:
-        out["roofline"] = roofline_of(m, n, k, bound, med, issue_peak_tops)
+        out["roofline"] = roofline_of(m, n, k, bound, med, issue_peak_tops, name=name, config=config)
     return out, (ap, bp, a_d, b_d, c_d)
 
 
@@ -238,6 +293,7 @@ def extras_4096(a_d, b_d, c_d):
     import torch
 
     import quadmul
+    import quadmul_amd as qm
 
     m = n = k = 4096
     dev = a_d.device
@@ -258,13 +314,13 @@ def extras_4096(a_d, b_d, c_d):
                                "ms_per_launch": round(s_ms, 5), "tops": round(2.0 * m * n * k / s_ms / 1e9, 1),
                                "frac_of_int8_peak": round(2.0 * m * n * k / s_ms / 1e9 / INT8_PEAK_TOPS, 4),
                                "algorithmic_bytes": m * k // 2 + n * k // 2 + 2 * m * n + 4 * (m + n),
-                               "traffic": PROFILED_TRAFFIC_OTHER["scaled_fp16_4096^3"],
+                               "traffic": profiled_traffic("square4096_scaled_f16", m, n, k, qm.config_name(qm.select_config_ex(m, n, k, scaled=True) & 0xFFFF))[0],
                                "checked": "every element against torch's float32 arithmetic on the int32 result"},
         "quantize_pack_fp16": {"entry_point": "quadmul.quantize_pack(x)", "rows": m, "k": k, "ms_per_launch": round(q_ms, 5),
                                "algorithmic_bytes": q_bytes,
                                "roofline": {"bound": "hbm", "achieved": round(q_bytes / q_ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                             "frac": round(q_bytes / q_ms / 1e6 / HBM_PEAK_GBS, 4),
-                                            "traffic": PROFILED_TRAFFIC_OTHER["quantize_pack_fp16_4096x4096"]}},
+                                            "traffic": profile_total("quantize4096_f16")}},
     }
 
 
@@ -319,6 +375,26 @@ def _timed(fn):
     return time.perf_counter() - t0
 
 
+def rotating_call(a_d, b_d, c_d, m, n, k):
+    """A call that rotates over enough copies of B (each with a C of its own) to exceed the
+    256 MiB memory-side cache, so that B comes from HBM: (callable, copies, the outputs)."""
+    import torch
+
+    import quadmul
+
+    ncopies = max(2, -(-(320 << 20) // max(1, b_d.numel())))
+    bs = [b_d] + [b_d.clone() for _ in range(ncopies - 1)]
+    cs = [c_d] + [torch.empty_like(c_d) for _ in range(ncopies - 1)]
+    turn = [0]
+
+    def fn_rot():
+        i = turn[0] % ncopies
+        turn[0] += 1
+        quadmul.gemm(a_d, bs[i], cs[i], m, n, k)
+
+    return fn_rot, ncopies, cs
+
+
 def launches_only(a):
     """Profiling aid: just N launches of one workload (after one warm-up), nothing else."""
     import torch
@@ -343,10 +419,13 @@ def launches_only(a):
         apk, bpk = make_packed(m, n, k, SEED_BASE + row)
         a_d, b_d = apk.to(dev), bpk.to(dev)
         c_d = torch.empty((m, n), dtype=torch.int32, device=dev)
+        fn = lambda: quadmul.gemm(a_d, b_d, c_d, m, n, k)
+        if a.rotate_b:
+            fn, _, _ = rotating_call(a_d, b_d, c_d, m, n, k)
         for _ in range(a.launches_only + 1):
-            quadmul.gemm(a_d, b_d, c_d, m, n, k)
+            fn()
     torch.cuda.synchronize()
-    print(json.dumps({"launches_only": a.launches_only, "workload": a.workload}))
+    print(json.dumps({"launches_only": a.launches_only, "workload": a.workload, "rotate_b": bool(a.rotate_b)}))
     return 0
 
 
@@ -357,6 +436,9 @@ def main(argv=None):
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS) + ["square4096_scaled_f16", "quantize4096_f16"],
                     help="the workload of the JSON line's value; the last two names exist for --launches-only (profiling) only")
+    ap.add_argument("--preheat-ms", type=float, default=400.0,
+                    help="untimed back-to-back launches of the headline kernel for this long before the warm-ups, so that the "
+                         "timed steps run at the sustained clock (0: none)")
     ap.add_argument("--no-targets", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-probes", action="store_true", help="skip the MFMA issue and launch floor probes")
@@ -364,6 +446,9 @@ def main(argv=None):
                     help="profiling aid: just N launches of --workload (after one warm-up), nothing else")
     ap.add_argument("--graph-only", type=int, default=0, metavar="N",
                     help="profiling aid: one HIP graph of N launches of --workload, replayed six times, nothing else")
+    ap.add_argument("--rotate-b", action="store_true",
+                    help="with --launches-only / --graph-only: the launches rotate over copies of B that exceed the memory-side "
+                         "cache, so that B comes from HBM")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: ten device-to-device copies of 256 MiB (a plain copy kernel of known "
                          "size, to scale the FETCH_SIZE / WRITE_SIZE counters)")
@@ -398,13 +483,27 @@ def main(argv=None):
         apk, bpk = make_packed(m, n, k, SEED_BASE + row)
         a_d, b_d = apk.to("cuda:0"), bpk.to("cuda:0")
         c_d = torch.empty((m, n), dtype=torch.int32, device="cuda:0")
-        med, lo, hi = time_graph(lambda: quadmul.gemm(a_d, b_d, c_d, m, n, k), launches=a.graph_only)
-        print(json.dumps({"graph_only": a.graph_only, "workload": a.workload, "ms_per_launch_median": round(med, 5),
+        fn = lambda: quadmul.gemm(a_d, b_d, c_d, m, n, k)
+        if a.rotate_b:
+            fn, _, _ = rotating_call(a_d, b_d, c_d, m, n, k)
+        med, lo, hi = time_graph(fn, launches=a.graph_only)
+        print(json.dumps({"graph_only": a.graph_only, "workload": a.workload, "rotate_b": bool(a.rotate_b), "ms_per_launch_median": round(med, 5),
                           "min_max": [round(lo, 5), round(hi, 5)]}))
         return 0
 
     import quadmul
     import quadmul_amd as qm
+
+    # every input is made and moved to the GPU before anything is timed: nothing but kernels
+    # runs between the probes and the timed steps
+    row, m, n, k, bound = WORKLOADS[a.workload]
+    apk, bpk = make_packed(m, n, k, SEED_BASE + row)
+    dev = torch.device("cuda:0")
+    a_d, b_d = apk.to(dev), bpk.to(dev)
+    c_d = torch.full((m, n), 0x7F7F7F7F, dtype=torch.int32, device=dev)
+    fn = lambda: quadmul.gemm(a_d, b_d, c_d, m, n, k)
+    fn()
+    torch.cuda.synchronize()
 
     probes = {}
     issue_peak = None
@@ -416,16 +515,10 @@ def main(argv=None):
         issue_peak = probes["mfma_issue_peak"]["tops"]
 
     # ---- the headline: exactly `steps` calls of quadmul.gemm after `warmup` untimed ones ----
-    row, m, n, k, bound = WORKLOADS[a.workload]
-    apk, bpk = make_packed(m, n, k, SEED_BASE + row)
-    dev = torch.device("cuda:0")
-    a_d, b_d = apk.to(dev), bpk.to(dev)
-    c_d = torch.full((m, n), 0x7F7F7F7F, dtype=torch.int32, device=dev)
-    fn = lambda: quadmul.gemm(a_d, b_d, c_d, m, n, k)
-    fn()
-    torch.cuda.synchronize()
-    wall_ms, event_ms = time_steps(fn, a.steps, a.warmup)
+    wall_ms, ev, pre = time_steps(fn, a.steps, a.warmup, a.preheat_ms)
+    event_ms = ev["mean"]
     graph_med, graph_lo, graph_hi = time_graph(fn, launches=int(min(2000, max(20, 50.0 / max(event_ms, 2e-3)))))
+    config = qm.config_name(qm.select_config(m, n, k) & 0xFFFF)
     line = {
         "metric": "int4 GEMM TOPS and % of int8 MFMA peak / % HBM BW, 1xMI355X",
         "value": round(2.0 * m * n * k / wall_ms / 1e9, 2), "unit": "TOPS", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -433,14 +526,18 @@ def main(argv=None):
         "vs_baseline": None,
         "dtype": "i8 (s4 nibbles widened to 16*s4) x i8 -> i32 MFMA, exact",
         "data": "synthetic",
-        "config": {"workload": workload_text(a.workload), "kernel": qm.config_name(qm.select_config(m, n, k) & 0xFFFF),
+        "config": {"workload": workload_text(a.workload), "kernel": config,
                    "entry_point": "quadmul.gemm(a, b, c, m, n, k)",
-                   "ms_per_step_events": round(event_ms, 5),
+                   # untimed launches of the same kernel before the warm-ups (see time_steps)
+                   "preheat_ms": pre["preheat_ms"], "preheat_launches": pre["preheat_launches"],
+                   "ms_per_step_events": round(event_ms, 5), "ms_per_step_events_median": round(ev["median"], 5),
+                   "ms_per_step_events_min_max": [round(ev["min"], 5), round(ev["max"], 5)],
                    "ms_per_launch_graph_median": round(graph_med, 5), "ms_per_launch_graph_min_max": [round(graph_lo, 5), round(graph_hi, 5)]},
         # average launch duration over the timed steps, from the HIP events around them
-        "roofline": roofline_of(m, n, k, bound, event_ms, issue_peak),
+        "roofline": roofline_of(m, n, k, bound, event_ms, issue_peak, name=a.workload, config=config),
     }
-    line["roofline"]["duration_source"] = f"HIP events around the {a.steps} timed steps on the launch stream, average per launch"
+    line["roofline"]["duration_source"] = (f"one HIP event per step on the launch stream: first to last over the {a.steps} timed steps, average per launch "
+                                           f"(after {pre['preheat_launches']} untimed launches = {pre['preheat_ms']} ms of the same kernel and {a.warmup} warm-ups)")
     line.update(probes)
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(apk, bpk, c_d, m, n, k)

@@ -45,8 +45,8 @@ def ext_path() -> str:
 
 # The compilers the full GPU suite has passed with.  The kernels order matrix-core
 # instructions and their hazards by hand inside asm statements; another compiler may schedule
-# the code around them differently, so a build with one is flagged until the suite has been
-# run on it (tests/ -m gpu is the gate).
+# the code around them differently, so a build with one is refused unless
+# QM_ALLOW_UNVALIDATED_COMPILER=1 says to go ahead (tests/ -m gpu is the gate for adding one).
 VALIDATED_COMPILERS = ("HIP version: 7.2",)
 
 
@@ -75,9 +75,15 @@ def build_lib(jobs: int = 8, verbose: bool = False) -> str:
     os.makedirs(OBJDIR, exist_ok=True)
     ver = compiler_version()
     if not any(ver.startswith(v) for v in VALIDATED_COMPILERS):
-        print(f"quadmul_amd.build: WARNING: building with {ver!r}, which the GPU test-suite has not been run with "
-              f"(validated: {', '.join(VALIDATED_COMPILERS)}); run `pytest tests -m gpu` before trusting results", file=sys.stderr)
-    units = [("qm_dispatch.o", [f'-DQM_COMPILER_VERSION="{ver}"', "-c", os.path.join(CSRC, "qm_dispatch.hip")])]
+        msg = (f"building with {ver!r}, which the GPU test-suite has not been run with "
+               f"(validated: {', '.join(VALIDATED_COMPILERS)})")
+        if os.environ.get("QM_ALLOW_UNVALIDATED_COMPILER") != "1":
+            raise RuntimeError(f"quadmul_amd.build: refusing: {msg}.  The kernels order matrix-core instructions and their "
+                               "hazards by hand; set QM_ALLOW_UNVALIDATED_COMPILER=1 to build anyway, then run "
+                               "`pytest tests -m gpu` before trusting any result and add the compiler to VALIDATED_COMPILERS")
+        print(f"quadmul_amd.build: WARNING: {msg}; run `pytest tests -m gpu` before trusting results", file=sys.stderr)
+    units = [("qm_dispatch.o", [f'-DQM_COMPILER_VERSION="{ver}"', "-c", os.path.join(CSRC, "qm_dispatch.hip")]),
+             ("qm_scratch.o", ["-c", os.path.join(CSRC, "qm_scratch.hip")])]
     for tu in range(N_TILE_TUS):
         units.append((f"qm_tile_inst_{tu}.o", [f"-DQM_TU={tu}", "-c", os.path.join(CSRC, "qm_tile_inst.hip")]))
     objs = [os.path.join(OBJDIR, name) for name, _ in units]

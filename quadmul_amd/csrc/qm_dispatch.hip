@@ -382,32 +382,6 @@ QM_EXPORT int qm_gemm_i4_ws(const void *A, const void *B, void *C, int m, int n,
     return run_gemm(A, B, C, m, n, k, nullptr, nullptr, OUT_I32, reinterpret_cast<hipStream_t>(stream), cfg, workspace, workspace_bytes);
 }
 
-// --------------------------------------------------------------------------
-// Library-owned scratch memory for qm_gemm_i4_static.  In host code the array's name is only
-// a handle for hipGetSymbolAddress: every device has its own copy at its own address, looked
-// up once per device (with that device current) and kept; kernels and every other use take
-// that pointer.
-// --------------------------------------------------------------------------
-static __device__ __align__(256) unsigned char scratch[QM_STATIC_SCRATCH_BYTES];
-static std::atomic<void *> g_scratch_ptr[QM_MAX_DEVICES] = {};
-
-static hipError_t static_scratch(void **out)
-{
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= QM_MAX_DEVICES) return hipErrorInvalidDevice;
-    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
-    if (ptr == nullptr) {
-        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-        if (e != hipSuccess) return e;
-        if (ptr == nullptr || ((uintptr_t)ptr & 255) != 0) return hipErrorInvalidSymbol;
-        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
-    }
-    *out = ptr;
-    return hipSuccess;
-}
-
 // Every one-off set-up a first launch on the current device would otherwise do.
 QM_EXPORT int qm_init(void)
 {

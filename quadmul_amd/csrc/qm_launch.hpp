@@ -48,6 +48,9 @@ inline hipError_t ensure_dynamic_lds(KernelPtr kernel, int bytes, std::atomic<bo
     return hipSuccess;
 }
 
+// The address, on the current device, of the library's own scratch array (qm_scratch.hip).
+hipError_t static_scratch(void **out);
+
 #define QM_SKINNY_FN(FM, FN, NW, U) qm_launch_skinny_##FM##_##FN##_##NW##_##U
 #define QM_DOT_FN(MR, FN, NW, U) qm_launch_dot_##MR##_##FN##_##NW##_##U
 #define QM_SKINNYD_FN(FM, FN, NW, D) qm_launch_skinnyd_##FM##_##FN##_##NW##_##D

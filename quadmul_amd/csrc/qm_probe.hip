@@ -7,7 +7,9 @@
 //   qm_probe_mfma_issue   a loop of independent v_mfma_i32_16x16x64_i8 on operands of the
 //                         form 16 * s4 (low nibble zero), the instruction and the operand
 //                         form of the GEMM kernels, with nothing else in the loop: the
-//                         issue peak of the matrix cores at the clock the part sustains
+//                         issue peak of the matrix cores at the clock the part sustains,
+//                         with every MFMA on the same operand registers or rotating over
+//                         four pairs of them
 //   qm_probe_empty        a kernel that does nothing: the launch floor
 //   qm_probe_read         a kernel that only reads `bytes` (16 bytes per lane, whole lines)
 //                         and keeps a checksum: the floor of "launch + one pass over B"
@@ -24,21 +26,27 @@ constexpr int MFMA_PER_ITER = 16;   // independent accumulators: 16 x 4 AGPRs
 constexpr int MFMA_OPS = 2 * 16 * 16 * 64;
 
 // One workgroup of four waves (one per SIMD) per launch slot; `iters` trips of 16 MFMAs.
+// PAIRS: distinct operand register pairs the MFMAs of a trip rotate over (1: every MFMA reads
+// the same two registers, so the operand buses never toggle -- an upper bound under a power
+// cap; 4: consecutive MFMAs read different pseudo-random operands, as the GEMM's do).
 // out[2 * block], out[2 * block + 1]: what the two counters of the core (s_memtime) and of
 // the constant 100 MHz reference (s_memrealtime) advanced by around the loop, from wave 0.
+template <int PAIRS>
 __global__ void __launch_bounds__(256) mfma_issue_kernel(uint64_t *out, int iters, uint32_t seed)
 {
     // pseudo-random nibbles in the high half of every byte: the matrix cores draw power by
     // the bits that toggle, so all-zero operands would flatter the result
     uint32_t h = (threadIdx.x + 1) * 2654435761u + blockIdx.x * 40503u + seed;
-    v4i s0, s1;
+    v4i s0[PAIRS], s1[PAIRS];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        h ^= h << 13; h ^= h >> 17; h ^= h << 5;
-        s0[i] = (int)(h & 0xF0F0F0F0u);
-        h ^= h << 13; h ^= h >> 17; h ^= h << 5;
-        s1[i] = (int)(h & 0xF0F0F0F0u);
-    }
+    for (int q = 0; q < PAIRS; ++q)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            h ^= h << 13; h ^= h >> 17; h ^= h << 5;
+            s0[q][i] = (int)(h & 0xF0F0F0F0u);
+            h ^= h << 13; h ^= h >> 17; h ^= h << 5;
+            s1[q][i] = (int)(h & 0xF0F0F0F0u);
+        }
     v4i acc[MFMA_PER_ITER];
 #pragma unroll
     for (int i = 0; i < MFMA_PER_ITER; ++i) acc[i] = v4i{0, 0, 0, 0};
@@ -46,7 +54,7 @@ __global__ void __launch_bounds__(256) mfma_issue_kernel(uint64_t *out, int iter
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
         for (int i = 0; i < MFMA_PER_ITER; ++i)
-            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(s0), "v"(s1));
+            asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(s0[i % PAIRS]), "v"(s1[i % PAIRS]));
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     const uint64_t t1 = __builtin_readcyclecounter(), r1 = wall_clock64();
@@ -82,12 +90,15 @@ __global__ void __launch_bounds__(1024) read_kernel(const v4i *src, size_t n16, 
 }  // namespace
 
 // Enqueues one launch of `blocks` workgroups x 4 waves x iters x 16 MFMAs.  out: device
-// memory for 2 * blocks uint64.  Returns the integer operations of the launch (2 * 16 * 16
-// * 64 per MFMA per wave) as a double, or a negative hipError_t.
-QM_PROBE_EXPORT double qm_probe_mfma_issue(void *out, int blocks, int iters, void *stream)
+// memory for 2 * blocks uint64.  operand_pairs: 1 or 4 (see the kernel).  Returns the integer
+// operations of the launch (2 * 16 * 16 * 64 per MFMA per wave) as a double, or a negative
+// hipError_t.
+QM_PROBE_EXPORT double qm_probe_mfma_issue(void *out, int blocks, int iters, int operand_pairs, void *stream)
 {
-    if (!out || blocks < 1 || iters < 1) return -1.0;
-    mfma_issue_kernel<<<dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream)>>>(static_cast<uint64_t *>(out), iters, 12345u);
+    if (!out || blocks < 1 || iters < 1 || (operand_pairs != 1 && operand_pairs != 4)) return -1.0;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (operand_pairs == 1) mfma_issue_kernel<1><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<uint64_t *>(out), iters, 12345u);
+    else mfma_issue_kernel<4><<<dim3(blocks), dim3(256), 0, s>>>(static_cast<uint64_t *>(out), iters, 12345u);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return -(double)(int)e;
     return (double)blocks * 4.0 * (double)iters * MFMA_PER_ITER * (double)MFMA_OPS;

@@ -3,7 +3,8 @@ what the part sustains, measured on the box, to set beside the nominal peaks.
 
     python -m quadmul_amd.probe          # prints one JSON object
 
-* ``mfma_issue_peak``: a loop of independent ``v_mfma_i32_16x16x64_i8`` on 16*s4 operands,
+* ``mfma_issue_peak``: a loop of independent ``v_mfma_i32_16x16x64_i8`` on 16*s4 operands
+  (rotating over four operand register pairs, and on one pair for comparison),
   nothing else in the loop, on every SIMD of the device, timed between two events like the
   reference's harness times its kernel (kernel.cu:468-497).  One such MFMA is 32768 integer
   operations and issues in 16 cycles of a SIMD, so the rate also gives the clock the part
@@ -34,7 +35,7 @@ def library() -> ctypes.CDLL:
             raise RuntimeError(f"{_LIB_PATH} is missing: build it with `python -m quadmul_amd.build`")
         lib = ctypes.CDLL(_LIB_PATH)
         vp, ci = ctypes.c_void_p, ctypes.c_int
-        lib.qm_probe_mfma_issue.argtypes = [vp, ci, ci, vp]
+        lib.qm_probe_mfma_issue.argtypes = [vp, ci, ci, ci, vp]
         lib.qm_probe_mfma_issue.restype = ctypes.c_double
         lib.qm_probe_empty.argtypes = [vp]
         lib.qm_probe_empty.restype = ci
@@ -44,22 +45,14 @@ def library() -> ctypes.CDLL:
     return _lib
 
 
-def mfma_issue_peak(seconds: float = 0.6, blocks_per_cu: int = 1):
-    """Sustained rate of the MFMA-only loop.  Launches of about 10 ms each, back to back
-    for `seconds` (long enough for the power management to settle), the last five timed
-    one by one: median."""
+def _mfma_issue_rate(lib, out, blocks, iters, pairs, seconds):
+    """(TOP/s, ms per launch, warm-up launches) of the MFMA-only loop on `pairs` operand register pairs."""
     import torch
 
-    lib = library()
-    dev = torch.device("cuda:0")
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    blocks = cus * blocks_per_cu
-    out = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
-    iters = 12000   # x 16 MFMAs x 16 cycles = 3.07 M cycles: about 1.3 ms at 2.4 GHz
 
     def launch():
-        ops = lib.qm_probe_mfma_issue(out.data_ptr(), blocks, iters, stream)
+        ops = lib.qm_probe_mfma_issue(out.data_ptr(), blocks, iters, pairs, stream)
         if ops < 0:
             raise RuntimeError(f"qm_probe_mfma_issue: hipError_t {int(-ops)}")
         return ops
@@ -83,7 +76,26 @@ def mfma_issue_peak(seconds: float = 0.6, blocks_per_cu: int = 1):
         e1.synchronize()
         times.append(e0.elapsed_time(e1))
     ms = statistics.median(times)
-    tops = ops / ms / 1e9
+    return ops / ms / 1e9, ms, n_warm
+
+
+def mfma_issue_peak(seconds: float = 0.6, blocks_per_cu: int = 1):
+    """Sustained rate of the MFMA-only loop.  Launches of about 1.3 ms each, back to back
+    for `seconds` (long enough for the power management to settle), the last five timed
+    one by one: median.  Measured twice: with consecutive MFMAs rotating over four pairs of
+    pseudo-random operand registers (``tops``: the operand buses toggle as they do in the
+    GEMM) and with every MFMA on one pair (``tops_one_operand_pair``: they do not, so under a
+    power cap this one is an upper bound)."""
+    import torch
+
+    lib = library()
+    dev = torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    blocks = cus * blocks_per_cu
+    out = torch.zeros(2 * blocks, dtype=torch.int64, device=dev)
+    iters = 12000   # x 16 MFMAs x 16 cycles = 3.07 M cycles: about 1.3 ms at 2.4 GHz
+    tops1, ms1, _ = _mfma_issue_rate(lib, out, blocks, iters, 1, seconds)
+    tops, ms, n_warm = _mfma_issue_rate(lib, out, blocks, iters, 4, seconds)
     counters = out.view(-1, 2).cpu()
     core, ref = int(counters[:, 0].max()), int(counters[:, 1].max())
     res = {
@@ -91,8 +103,13 @@ def mfma_issue_peak(seconds: float = 0.6, blocks_per_cu: int = 1):
         "frac_of_nominal_int8_peak": round(tops / INT8_PEAK_TOPS, 4),
         # 16 cycles per MFMA and SIMD, every SIMD of every CU busy: rate / nominal rate x 2.4 GHz
         "implied_clock_mhz": round(tops / (INT8_PEAK_TOPS * cus / 256.0) * NOMINAL_MHZ, 0),
-        "instruction": "v_mfma_i32_16x16x64_i8, operands 16*s4, 16 independent accumulators per wave, one wave per SIMD",
+        "instruction": "v_mfma_i32_16x16x64_i8, operands 16*s4, 16 independent accumulators per wave, one wave per SIMD, "
+                       "consecutive MFMAs on four different pairs of operand registers",
         "launch_ms_median_of_5": round(ms, 4), "warmup_launches": n_warm, "cus": cus,
+        "tops_one_operand_pair": round(tops1, 1),
+        "one_operand_pair": {"tops": round(tops1, 1), "frac_of_nominal_int8_peak": round(tops1 / INT8_PEAK_TOPS, 4),
+                             "launch_ms_median_of_5": round(ms1, 4),
+                             "note": "every MFMA reads the same two registers: the operand buses do not toggle (upper bound under a power cap)"},
         "method": "launches between two HIP events after the warm-ups (as kernel.cu:468-497)",
     }
     if ref > 0:
