@@ -11,6 +11,11 @@ the reference's ``benchmarks/a40.md``:
 
 Before timing, each shape is checked: the int4 result must equal the int8 library
 result exactly (the reference accepts |diff| <= 1, test.py:41-43).
+
+A second table times the same shapes through the bare seven-argument C entry point
+``qm_gemm_i4`` -- the function a maintainer binds in place of the reference's ``wrapper``
+(kernel.cu:334) -- which has no workspace to split K through, beside ``quadmul.gemm``, which
+takes one from torch's allocator.
 """
 from __future__ import annotations
 
@@ -42,11 +47,27 @@ def bench_shape(m: int, n: int, k: int, dev) -> dict:
     c_h = torch.empty((m, n), dtype=torch.float16, device=dev)
     t_i8 = time_launches(lambda: torch._int_mm(a, bt, out=c_ref), 20.0, 3)
     t_i4 = time_launches(lambda: quadmul.gemm(a_p, b_p, c, m, n, k), 20.0, 3)
+    # the bare C entry point: the same seven arguments as the reference's wrapper, no workspace
+    lib = qm.library()
+    c_bare = torch.full((m, n), 0x7F7F7F7F, dtype=torch.int32, device=dev)
+
+    def bare():
+        st = lib.qm_gemm_i4(a_p.data_ptr(), b_p.data_ptr(), c_bare.data_ptr(), m, n, k, torch.cuda.current_stream().cuda_stream)
+        if st != 0:
+            raise RuntimeError(f"qm_gemm_i4: status {st}")
+
+    bare()
+    torch.cuda.synchronize()
+    exact = exact and bool(torch.equal(c_bare, c_ref))
+    t_bare = time_launches(bare, 20.0, 3)
     t_f16 = time_launches(lambda: torch.matmul(a_h, b_h.t(), out=c_h), 20.0, 3)
     ops = 2.0 * m * n * k
     cfg = qm.select_config(m, n, k)
-    return {"m": m, "n": n, "k": k, "exact": exact, "kernel": qm.config_name(cfg & 0xFFFF),
-            "int8": ops / t_i8 / 1e9, "int4": ops / t_i4 / 1e9, "fp16": ops / t_f16 / 1e9}
+    cfg_bare = qm.select_config_ex(m, n, k, workspace=False)
+    return {"m": m, "n": n, "k": k, "exact": exact, "kernel": qm.config_name(cfg & 0xFFFF), "ksplit": max(1, (cfg >> 24) & 0x3F),
+            "kernel_bare": qm.config_name(cfg_bare & 0xFFFF), "ksplit_bare": max(1, (cfg_bare >> 24) & 0x3F),
+            "int8": ops / t_i8 / 1e9, "int4": ops / t_i4 / 1e9, "fp16": ops / t_f16 / 1e9, "int4_bare": ops / t_bare / 1e9,
+            "us": t_i4 * 1e3, "us_bare": t_bare * 1e3}
 
 
 def main(argv=None) -> int:
@@ -83,6 +104,22 @@ def main(argv=None) -> int:
         lines.append(f"| {r['m']} | {r['n']} | {r['k']} | {r['int8']:.2f} | {r['int4']:.2f} | {r['fp16']:.2f} | "
                      f"{r['int4']/r['int8']:.2f}x | {r['int4']/r['fp16']:.2f}x | {100*r['int4']/INT8_PEAK_TOPS:.1f} | "
                      f"{'yes' if r['exact'] else 'NO'} | {r['kernel']} |")
+    lines += [
+        "",
+        "### The same shapes through the bare entry point `qm_gemm_i4(A, B, C, m, n, k, stream)`",
+        "",
+        "`qm_gemm_i4` takes the seven arguments of the reference's `wrapper` (kernel.cu:334) and nothing else, so it has no "
+        "workspace: where the table above splits K through one (K split > 1 there), it runs the cost model's choice without, "
+        "partial sums meeting in C through integer atomics if it splits at all.  Same operands, same timing method, results "
+        "checked bit-exact.  `qm_gemm_i4_ws` (a caller's workspace) and `qm_gemm_i4_static` (the library's own scratch array) "
+        "run what `quadmul.gemm` runs.",
+        "",
+        "| M | N | K | quadmul.gemm us | K split | qm_gemm_i4 us | K split | qm_gemm_i4 / quadmul.gemm | qm_gemm_i4 TOP/s | kernel |",
+        "|---|---|---|---|---|---|---|---|---|---|",
+    ]
+    for r in rows:
+        lines.append(f"| {r['m']} | {r['n']} | {r['k']} | {r['us']:.1f} | {r['ksplit']} | {r['us_bare']:.1f} | {r['ksplit_bare']} | "
+                     f"{r['us_bare']/r['us']:.2f}x | {r['int4_bare']:.2f} | {r['kernel_bare']} |")
     text = "\n".join(lines) + "\n"
     if a.out:
         with open(a.out, "w") as f:

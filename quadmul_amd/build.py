@@ -82,7 +82,7 @@ def build_lib(jobs: int = 8, verbose: bool = False) -> str:
                                "hazards by hand; set QM_ALLOW_UNVALIDATED_COMPILER=1 to build anyway, then run "
                                "`pytest tests -m gpu` before trusting any result and add the compiler to VALIDATED_COMPILERS")
         print(f"quadmul_amd.build: WARNING: {msg}; run `pytest tests -m gpu` before trusting results", file=sys.stderr)
-    units = [("qm_dispatch.o", [f'-DQM_COMPILER_VERSION="{ver}"', "-c", os.path.join(CSRC, "qm_dispatch.hip")]),
+    units = [("qm_dispatch.o", [f'-DQM_COMPILER_VERSION="{ver}"', "-mllvm", "-amdgpu-kernarg-preload-count=16", "-c", os.path.join(CSRC, "qm_dispatch.hip")]),
              ("qm_scratch.o", ["-c", os.path.join(CSRC, "qm_scratch.hip")])]
     for tu in range(N_TILE_TUS):
         units.append((f"qm_tile_inst_{tu}.o", [f"-DQM_TU={tu}", "-c", os.path.join(CSRC, "qm_tile_inst.hip")]))

@@ -111,6 +111,12 @@ __device__ __forceinline__ v4i mfma16(const v4i s0, const v4i s1, const v4i acc)
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(s0, s1, acc, 0, 0, 0);
 }
 
+// Byte offset of row `row` of a packed operand with Kb bytes per row, for the skinny
+// kernels: both factors are below 2^24 there (the host side sees to it), so the full-rate
+// 24-bit multiply does (the 32-bit one issues at a quarter of the rate, and these products
+// sit in front of a wave's first load).
+__device__ __forceinline__ uint32_t row_bytes24(int row, int Kb) { return __umul24((uint32_t)row, (uint32_t)Kb); }
+
 // Workgroups are dealt round-robin to the 8 XCDs (id % 8), each with a private
 // L2.  Renumber so that every XCD owns one contiguous range of tile ids.
 __device__ __forceinline__ int xcd_contiguous_id(int bid, int nblocks)

@@ -46,7 +46,7 @@ static hipError_t launch_dot(const GemmArgs &p, hipStream_t stream, int opt)
 {
     if (opt & QM_OPT_PREPARE) return hipSuccess;
     const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
-    gemm_dot_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), 0, stream>>>(p);
+    gemm_dot_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), 0, stream>>>(p.A, p.B, p.C, p.M, p.N, p.K, p.ldc, p.out, p.row_scale, p.col_scale);
     return hipGetLastError();
 }
 #define QM_DOT(MR, FN, NW, U) \
@@ -58,8 +58,9 @@ static hipError_t launch_skinny_dma(const GemmArgs &p, hipStream_t stream, int o
     const hipError_t e = ensure_dynamic_lds(&gemm_skinny_dma_kernel<Cfg>, Cfg::LDS_BYTES, lds_ok);
     if (e != hipSuccess) return e;
     if (opt & QM_OPT_PREPARE) return hipSuccess;
-    const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
-    gemm_skinny_dma_kernel<Cfg><<<dim3(blocks), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p);
+    const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN, row_blocks = (p.M + Cfg::MAX_M - 1) / Cfg::MAX_M;
+    if (row_blocks > 65535) return hipErrorInvalidValue;
+    gemm_skinny_dma_kernel<Cfg><<<dim3(blocks, row_blocks), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p.A, p.B, p.C, p.M, p.N, p.K, p.ldc, p.out, p.row_scale, p.col_scale);
     return hipGetLastError();
 }
 // Compute units of the current device (asked once per device).
@@ -92,7 +93,9 @@ static hipError_t launch_skinny_stream_dma(const GemmArgs &p, hipStream_t stream
     if (opt & QM_OPT_PREPARE) return hipSuccess;
     const int blocks = (p.N + Cfg::BN - 1) / Cfg::BN;
     const int resident = cus * (160 * 1024 / Cfg::LDS_BYTES);  // workgroups the device holds at once (the LDS decides)
-    gemm_skinny_stream_dma_kernel<Cfg><<<dim3(blocks < resident ? blocks : resident), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(p, blocks);
+    const int grid = blocks < resident ? blocks : resident;
+    gemm_skinny_stream_dma_kernel<Cfg><<<dim3(grid), dim3(Cfg::THREADS), Cfg::LDS_BYTES, stream>>>(
+        p.A, p.B, p.C, p.M, p.N, p.K, p.ldc, p.out | (grid << 8), blocks, p.row_scale, p.col_scale);
     return hipGetLastError();
 }
 #define QM_SKINNYP(FM, FN, NW, D, R) \

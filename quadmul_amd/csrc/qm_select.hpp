@@ -18,11 +18,12 @@ enum Kind { KIND_GENERIC = 0, KIND_SKINNY = 2, KIND_TILE16 = 3 };
 struct ConfigDesc {
     const char *name;
     int kind;
-    int bm, bn, bk;  // tile: block shape; skinny: bm = max M, bn = columns per workgroup
+    int bm, bn, bk;  // tile: block shape; skinny: bm = rows, bn = columns per workgroup (bm is the most M takes, without row_blocks)
     int waves, mode;
     LaunchFn launch;
     int wgm = 0, wgn = 0;  // pipelined kernel: waves down and across the tile
     int max_k = 0;         // skinny kernels whose waves hold A in registers: the K they hold (0: any)
+    bool row_blocks = false;  // skinny kernels whose grid walks over blocks of bm rows: any M
 };
 
 #define QM_STR2(x) #x
@@ -37,7 +38,7 @@ static const ConfigDesc g_configs[] = {
      &QM_SKINNY_FN(FM, FN, NW, U)},
 #define QM_SKINNYD(FM, FN, NW, D)                                                    \
     {"d" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_r" QM_STR(D), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
-     &QM_SKINNYD_FN(FM, FN, NW, D)},
+     &QM_SKINNYD_FN(FM, FN, NW, D), 0, 0, 0, true},
 #define QM_SKINNYP(FM, FN, NW, D, R)                                                 \
     {"p" QM_STR(FM) "x" QM_STR(FN) "_w" QM_STR(NW) "_r" QM_STR(D) "k" QM_STR(R), KIND_SKINNY, 16 * (FM), 16 * (FN), 128, NW, 0, \
      &QM_SKINNYP_FN(FM, FN, NW, D, R), 0, 0, 256 * (NW) * (R)},
@@ -90,7 +91,9 @@ static bool config_supports(int cfg, int m, int n, int k, int ptr_align)
     const ConfigDesc &c = g_configs[cfg];
     if (c.kind == KIND_GENERIC) return true;
     if (!fast_path_ok(m, n, k, ptr_align)) return false;
-    if (c.kind == KIND_SKINNY) return m <= c.bm && (c.max_k == 0 || k <= c.max_k);
+    // (the skinny kernels address rows through 24-bit multiplies: rows and bytes per row below 2^24)
+    if (c.kind == KIND_SKINNY)
+        return (m <= c.bm || (c.row_blocks && m <= 65535 * c.bm)) && (c.max_k == 0 || k <= c.max_k) && m < (1 << 24) && n < (1 << 24) && k / 2 < (1 << 24);
     if (c.kind == KIND_TILE16) return k % 128 == 0 || k > 128;  // a short last K-step needs a step before it
     return true;
 }
@@ -121,6 +124,8 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
     // Up to 64 rows: chosen on measurements with B streamed from HBM (launches rotating over
     // copies of B), M = 1 .. 64, N = 2048 .. 28672, K = 2048 .. 14336.
     const auto pick = [](const char *name) { const int id = find_config(name); return Choice{id >= 0 ? id : 0, 1, 1}; };
+    const bool skinny_ok = m < (1 << 24) && n < (1 << 24);  // (their 24-bit row arithmetic, see config_supports)
+    if (!skinny_ok) goto tiles;
     if (m <= 2) {
         // no matrix core: v_dot8_i32_i4 on the packed bytes as they are
         if (m == 1) return pick(k <= 2048 ? "v1x1_w8_u4" : (k <= 4096 ? "v1x1_w4_u8" : "v1x1_w16_u2"));
@@ -135,13 +140,30 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
     }
     if (m <= 32) {
         if (k <= 2048) return pick("p2x1_w16_r2k1");
+        // few column blocks and a long K: two blocks of 16 rows each double the workgroups
+        if (n <= 2048) return pick("d1x1_w16_r1");
         if (k <= 4096) return pick("p2x1_w8_r2k2");
-        // (a long K on many columns: every workgroup re-reads all of A, which the
-        // register-staged form does with fewer, larger loads)
-        return pick(n <= 8192 ? "d2x1_w16_r1" : "s2x1_w16_u2");
+        // a long K: every workgroup re-reads the rows of A it owns over all of K; 32 columns
+        // per workgroup halve that against 16
+        return pick(n <= 4096 ? "d2x1_w16_r1" : "d2x2_w8_r1");
     }
-    if (m <= 64 && n <= 8192) return pick("d4x1_w8_r1");
-    if (m <= 64 && n <= 16384 && config_supports(find_config("q64x64_w2x2_s8o2"), m, n, k, ptr_align)) return pick("q64x64_w2x2_s8o2");
+    if (m <= 64) {
+        // blocks of 32 rows: 32 x 16 per workgroup while that leaves one workgroup per CU,
+        // 32 x 32 (two to a CU) up to about three rounds of them, tiles beyond
+        if (n <= 2048) return pick("d2x1_w16_r1");
+        if (n <= 12288) return pick("d2x2_w8_r1");
+        if (n <= 16384 && config_supports(find_config("q64x64_w2x2_s8o2"), m, n, k, ptr_align)) return pick("q64x64_w2x2_s8o2");
+    }
+    if (m <= 256 && k <= 16384) {
+        // The same 32 x 32 blocks on a few hundred rows (measured with B from HBM, M = 65 .. 256,
+        // N = 2048 .. 11008, K = 2048 .. 8192): ahead of the tiles -- no ring to fill, one
+        // workgroup per 32 x 32 block of C over all of K -- up to about three rounds of
+        // workgroups (two to a CU), e.g. 128 x 4096 x 8192 11.4 us against 17.3, 192 x 4096 x 4096
+        // 9.7 against 11.1; level with the 64 x 64 tiles at four rounds, behind them beyond.
+        const long long wgs = (long long)((m + 31) / 32) * ((n + 31) / 32);
+        if (wgs <= 800 || (wgs <= 1040 && m <= 96)) return pick("d2x2_w8_r1");
+    }
+tiles:
     // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency),
     // over the configurations that can run this K.  Efficiencies are measured ratios.
     // eff: throughput per tile area relative to the 256 x 256 tile with the GPU full (measured)
@@ -185,7 +207,7 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         }
         if (cost < best_cost) { best_cost = cost; best = id; best_ks = ks; }
     }
-    if (m <= 128) {
+    if (m <= 128 && skinny_ok) {
         // The wave-level split-K kernel has no ring to fill and no second kernel, and wins
         // while N x K is small.  Measured, in the units above: about 2 us plus, per million
         // elements of B, 0.24 us with four row blocks (33..64 rows, B from HBM) and 0.38 us

@@ -110,9 +110,9 @@ gemm_skinny_kernel(const GemmArgs p)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
 #pragma unroll
-            for (int j = 0; j < FN; ++j) b8_off[j][h] = (uint32_t)min(n0 + j * 16 + 8 * h + ld8_row, p.N - 1) * (uint32_t)Kb + ld8_ch * 16;
+            for (int j = 0; j < FN; ++j) b8_off[j][h] = row_bytes24(min(n0 + j * 16 + 8 * h + ld8_row, p.N - 1), Kb) + ld8_ch * 16;
 #pragma unroll
-            for (int i = 0; i < FM; ++i) a8_off[i][h] = (uint32_t)min(i * 16 + 8 * h + ld8_row, p.M - 1) * (uint32_t)Kb + ld8_ch * 16;
+            for (int i = 0; i < FM; ++i) a8_off[i][h] = row_bytes24(min(i * 16 + 8 * h + ld8_row, p.M - 1), Kb) + ld8_ch * 16;
         }
         for (int c0 = wave * U; c0 < nchunks; c0 += NW * U) {
             v4i bl[U / 2][FN][2], al[U / 2][FM][2];
@@ -147,9 +147,9 @@ gemm_skinny_kernel(const GemmArgs p)
         const int from_lane = (4 * r + g) * 4;  // where MFMA lane (r, g) finds its fragment (byte address of a lane)
         uint32_t b_off[FN], a_off[FM];
 #pragma unroll
-        for (int j = 0; j < FN; ++j) b_off[j] = (uint32_t)min(n0 + j * 16 + ld_row, p.N - 1) * (uint32_t)Kb + ld_ch * 16;
+        for (int j = 0; j < FN; ++j) b_off[j] = row_bytes24(min(n0 + j * 16 + ld_row, p.N - 1), Kb) + ld_ch * 16;
 #pragma unroll
-        for (int i = 0; i < FM; ++i) a_off[i] = (uint32_t)min(i * 16 + ld_row, p.M - 1) * (uint32_t)Kb + ld_ch * 16;
+        for (int i = 0; i < FM; ++i) a_off[i] = row_bytes24(min(i * 16 + ld_row, p.M - 1), Kb) + ld_ch * 16;
         for (int c0 = wave * U; c0 < nchunks; c0 += NW * U) {
             v4i bq[U][FN], aq[U][FM];
 #pragma unroll
@@ -230,7 +230,7 @@ gemm_skinny_stream_kernel(const GemmArgs p, const int nblocks)
         for (int j = 0; j < FN; ++j)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const uint32_t row = (uint32_t)min(blk * Cfg::BN + j * 16 + 8 * h + ld8_row, p.N - 1) * (uint32_t)Kb;
+                const uint32_t row = row_bytes24(min(blk * Cfg::BN + j * 16 + 8 * h + ld8_row, p.N - 1), Kb);
 #pragma unroll
                 for (int pu = 0; pu < PAIRS; ++pu)
                     bl[pu][j][h] = ok[pu] ? __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p.B + row + kofs[pu])) : v4i{0, 0, 0, 0};
@@ -246,7 +246,7 @@ gemm_skinny_stream_kernel(const GemmArgs p, const int nblocks)
         v4i al[PAIRS][2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const uint32_t row = (uint32_t)min(i * 16 + 8 * h + ld8_row, p.M - 1) * (uint32_t)Kb;
+            const uint32_t row = row_bytes24(min(i * 16 + 8 * h + ld8_row, p.M - 1), Kb);
 #pragma unroll
             for (int pu = 0; pu < PAIRS; ++pu)
                 al[pu][h] = ok[pu] ? *reinterpret_cast<const v4i *>(p.A + row + kofs[pu]) : v4i{0, 0, 0, 0};
@@ -341,8 +341,15 @@ struct DotCfg {
 
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS)
-gemm_dot_kernel(const GemmArgs p)
+gemm_dot_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int M, const int N, const int K, const int ldc, const int out,
+                       const float *row_scale, const float *col_scale)
 {
+    // (scalar arguments: preloaded into SGPRs before the first wave starts, see gemm_skinny_stream_dma_kernel)
+    GemmArgs p{A, B, C, M, N, K};
+    p.row_scale = row_scale;
+    p.col_scale = col_scale;
+    p.out = out;
+    p.ldc = ldc;
     constexpr int MR = Cfg::MR, FN = Cfg::FN, NW = Cfg::NW, U = Cfg::U;
     __shared__ int32_t red[MR][FN * 16];  // the sum over the waves
 
@@ -358,9 +365,9 @@ gemm_dot_kernel(const GemmArgs p)
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) b_off[j][h] = (uint32_t)min(n0 + j * 16 + 8 * h + ld_row, p.N - 1) * (uint32_t)Kb + ld_ch * 16;
+        for (int h = 0; h < 2; ++h) b_off[j][h] = row_bytes24(min(n0 + j * 16 + 8 * h + ld_row, p.N - 1), Kb) + ld_ch * 16;
 #pragma unroll
-    for (int i = 0; i < MR; ++i) a_off[i] = (uint32_t)min(i, p.M - 1) * (uint32_t)Kb + ld_ch * 16;
+    for (int i = 0; i < MR; ++i) a_off[i] = row_bytes24(min(i, p.M - 1), Kb) + ld_ch * 16;
 
     int32_t acc[MR][FN][2];
 #pragma unroll

@@ -27,9 +27,18 @@
 //
 // Every wave owns its ring slots (its own runs of K): no barrier between loading and
 // contracting, only the wave's own s_waitcnt.  The waves' partial blocks are added up in
-// the LDS with integer atomics; the wave that arrives last (an LDS counter) reads the sums
-// and stores C, 16 bytes per lane.  One launch, no workspace, no global atomics, C
+// the LDS with integer atomics; after one barrier the waves read the sums and store C, one
+// 16 x 16 block per wave, 16 bytes per lane.  One launch, no workspace, no global atomics, C
 // overwritten.
+//
+// Rows beyond 16 FM: the grid's second dimension walks over blocks of 16 FM rows of A
+// (blockIdx.y), so a workgroup owns 16 FM rows x 16 FN columns.  Every workgroup pulls the
+// rows of A and of B it owns through its CU's L1 once, over all of K: with four fragment
+// blocks a square 2 x 2 moves 4 runs per 128 bytes of K where 4 x 1 moves 5, and its ring
+// slot is 8 KiB instead of 10, so that two runs per wave -- all of K = 4096 on eight waves --
+// are in flight at once within the 160 KiB of LDS.  The workgroups of one column block lie
+// gridDim.x apart in launch order, on the same XCD when gridDim.x is a multiple of 8: the
+// second reader of B's lines finds them in that XCD's L2.
 #pragma once
 #include <type_traits>
 
@@ -46,7 +55,7 @@ struct SkinnyDmaCfg {
     static constexpr int SLOT_BYTES = BLOCKS * 2048;   // one run of every block: 2 loads of 1 KiB each
     static constexpr int RING_BYTES = NW * D * SLOT_BYTES;
     static constexpr int RED_BYTES = FM * FN * 1024;   // the sum of the waves' blocks: [block][register][lane]
-    static constexpr int LDS_BYTES = RING_BYTES + RED_BYTES + 16;
+    static constexpr int LDS_BYTES = RING_BYTES + RED_BYTES;
     static constexpr int LOADS_PER_RUN = 2 * BLOCKS;
     static_assert(D >= 1 && D <= 4, "ring depth");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU");
@@ -55,17 +64,24 @@ struct SkinnyDmaCfg {
 
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS)
-gemm_skinny_dma_kernel(const GemmArgs p)
+gemm_skinny_dma_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int M, const int N, const int K, const int ldc, const int out,
+                       const float *row_scale, const float *col_scale)
 {
+    // (scalar arguments: preloaded into SGPRs before the first wave starts, see gemm_skinny_stream_dma_kernel)
+    GemmArgs p{A, B, C, M, N, K};
+    p.row_scale = row_scale;
+    p.col_scale = col_scale;
+    p.out = out;
+    p.ldc = ldc;
     constexpr int FM = Cfg::FM, FN = Cfg::FN, NW = Cfg::NW, D = Cfg::D, LPR = Cfg::LOADS_PER_RUN;
     extern __shared__ __align__(16) uint8_t smem[];
     int32_t *const red = reinterpret_cast<int32_t *>(smem + Cfg::RING_BYTES);
-    int *const arrived = reinterpret_cast<int *>(smem + Cfg::RING_BYTES + Cfg::RED_BYTES);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * Cfg::BN;
+    const int n0 = blockIdx.x * Cfg::BN, m0 = blockIdx.y * Cfg::MAX_M;
+    const bool b_read_once = M <= Cfg::MAX_M;  // one block of rows (gridDim.y == 1, without fetching the grid's size)
     const int Kb = p.K >> 1;             // bytes per row; a multiple of 16
     const int nruns = (Kb + 127) >> 7;   // 128-byte runs per row, the last one possibly short
     // this wave's runs: wave, wave + NW, ...
@@ -82,9 +98,9 @@ gemm_skinny_dma_kernel(const GemmArgs p)
         const int r16 = 8 * h + row8;
         piece_off[h] = (uint32_t)((pos ^ ((r16 >> 1) & 7)) * 16);
 #pragma unroll
-        for (int i = 0; i < FM; ++i) row_off[i][h] = (uint32_t)min(i * 16 + r16, p.M - 1) * (uint32_t)Kb;
+        for (int i = 0; i < FM; ++i) row_off[i][h] = row_bytes24(min(m0 + i * 16 + r16, p.M - 1), Kb);
 #pragma unroll
-        for (int j = 0; j < FN; ++j) row_off[FM + j][h] = (uint32_t)min(n0 + j * 16 + r16, p.N - 1) * (uint32_t)Kb;
+        for (int j = 0; j < FN; ++j) row_off[FM + j][h] = row_bytes24(min(n0 + j * 16 + r16, p.N - 1), Kb);
     }
     const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
     const uint32_t wave_lds = __builtin_amdgcn_readfirstlane(lds0 + wave * D * Cfg::SLOT_BYTES);
@@ -96,10 +112,12 @@ gemm_skinny_dma_kernel(const GemmArgs p)
             for (int h = 0; h < 2; ++h) {
                 const uint32_t dst = wave_lds + slot * Cfg::SLOT_BYTES + (2 * b + h) * 1024;
                 const uint32_t goff = row_off[b][h] + min((uint32_t)run * 128u + piece_off[h], last16);
-                // (B is read once and streams from HBM: marked non-temporal, it does not push
-                // A out of the L2s -- measured 5-10 % on shapes whose B exceeds them)
+                // (a B that is read once and streams from HBM is marked non-temporal: it does not
+                // push A out of the L2s -- measured 5-10 % on shapes whose B exceeds them; with
+                // several row blocks the later readers want its lines kept)
                 if (b < FM) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(goff), "s"(p.A) : "memory", "m0");
-                else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff), "s"(p.B) : "memory", "m0");
+                else if (b_read_once) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff), "s"(p.B) : "memory", "m0");
+                else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(goff), "s"(p.B) : "memory", "m0");
             }
     };
 
@@ -111,7 +129,6 @@ gemm_skinny_dma_kernel(const GemmArgs p)
     // (the sums start from zero; cleared while the loads are in flight, and the barrier comes
     // while every wave is still waiting for its data anyway)
     for (int idx = tid; idx < FM * FN * 256; idx += Cfg::THREADS) red[idx] = 0;
-    if (tid == 0) *arrived = 0;
     __syncthreads();
 
     // ---- reader side: lane (r, g) of a fragment, chunk j of the run -> logical piece 4 j + g ----
@@ -198,53 +215,45 @@ gemm_skinny_dma_kernel(const GemmArgs p)
                 for (int e = 0; e < 4; ++e)
                     __hip_atomic_fetch_add(&red[((i * FN + j) * 4 + e) * 64 + lane], acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    // The wave that arrives last stores.  A wave's LDS instructions are carried out in the
-    // order it issued them and its adds are complete before it takes its ticket, so the
-    // wave that draws the last ticket finds every wave's adds done.
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    int ticket = 0;
-    if (lane == 0) ticket = __hip_atomic_fetch_add(arrived, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    ticket = __builtin_amdgcn_readfirstlane(ticket);
-    if (ticket != NW - 1) return;
+    // Every wave's adds are complete at the barrier; block bb is then stored by wave bb % NW.
+    __syncthreads();
 
-    // lane (r, g) of block (i, j) holds C[16 i + r][n0 + 16 j + 4 g .. + 3]
+    // lane (r, g) of block (i, j) holds C[m0 + 16 i + r][n0 + 16 j + 4 g .. + 3]
     const bool vec_ok = (c_stride(p) & 3) == 0 && ((uintptr_t)p.C & (p.out == OUT_I32 ? 15 : 7)) == 0;
+    for (int bb = wave; bb < FM * FN; bb += NW) {
+        const int i = bb / FN, j = bb % FN;
+        v4i s;
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            v4i s;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) s[e] = red[((i * FN + j) * 4 + e) * 64 + lane] >> 8;
-            const int m = i * 16 + r, n = n0 + j * 16 + 4 * g;
-            if (m >= p.M || n >= p.N) continue;
-            const size_t at = (size_t)m * c_stride(p) + n;
-            if (p.out == OUT_I32) {
-                if (vec_ok) {
-                    *reinterpret_cast<v4i *>(p.C + at) = s;  // n % 4 == 0 and N % 4 == 0 (with a row stride: N is that stride or differs from it by a multiple of 256): all four inside
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < p.N) p.C[at + e] = s[e];
-                }
+        for (int e = 0; e < 4; ++e) s[e] = red[(bb * 4 + e) * 64 + lane] >> 8;
+        const int m = m0 + i * 16 + r, n = n0 + j * 16 + 4 * g;
+        if (m >= p.M || n >= p.N) continue;
+        const size_t at = (size_t)m * c_stride(p) + n;
+        if (p.out == OUT_I32) {
+            if (vec_ok) {
+                *reinterpret_cast<v4i *>(p.C + at) = s;  // n % 4 == 0 and N % 4 == 0 (with a row stride: N is that stride or differs from it by a multiple of 256): all four inside
             } else {
-                uint16_t *const d = reinterpret_cast<uint16_t *>(p.C) + at;
-                const float rs = scale_at(p.row_scale, m, p.M);
-                uint16_t h[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int c = s[e];
-                    h[e] = round16(scaled(c, rs, scale_at(p.col_scale, n + e, p.N)), p.out);
-                }
-                if (vec_ok) {
-                    *reinterpret_cast<v2i *>(d) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
-                } else {
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < p.N) p.C[at + e] = s[e];
+            }
+        } else {
+            uint16_t *const d = reinterpret_cast<uint16_t *>(p.C) + at;
+            const float rs = scale_at(p.row_scale, m, p.M);
+            uint16_t h[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < p.N) d[e] = h[e];
-                }
+            for (int e = 0; e < 4; ++e) {
+                const int c = s[e];
+                h[e] = round16(scaled(c, rs, scale_at(p.col_scale, n + e, p.N)), p.out);
+            }
+            if (vec_ok) {
+                *reinterpret_cast<v2i *>(d) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < p.N) d[e] = h[e];
             }
         }
+    }
 }
 
 }  // namespace qm
@@ -280,10 +289,23 @@ struct SkinnyStreamCfg {
     static_assert(R * FM * 16 <= 64, "A's widened fragments live in registers");
 };
 
+// (The arguments are scalars, not a GemmArgs by value: scalar kernel arguments are preloaded
+// into SGPRs before the first wave starts -- the library is built with
+// -amdgpu-kernarg-preload-count=16 -- where a structure is fetched by the waves themselves;
+// measured 1.5 % at M = 16, N = K = 4096 with B from HBM.)
 template <class Cfg>
 __global__ void __launch_bounds__(Cfg::THREADS)
-gemm_skinny_stream_dma_kernel(const GemmArgs p, const int nblocks)
+gemm_skinny_stream_dma_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int M, const int N, const int K, const int ldc,
+                              const int out_and_grid, const int nblocks, const float *row_scale, const float *col_scale)  // 16 dwords: all preloaded
 {
+    // (out_and_grid: the output form in bits 0..7, the number of workgroups above.  gridDim.x
+    // is a hidden kernel argument beyond the preloaded ones: read from there it is a scalar
+    // load that every wave waits for before it can issue its first load.)
+    GemmArgs p{A, B, C, M, N, K};
+    p.row_scale = row_scale;
+    p.col_scale = col_scale;
+    p.out = out_and_grid & 0xFF;
+    p.ldc = ldc;
     constexpr int FM = Cfg::FM, FN = Cfg::FN, NW = Cfg::NW, D = Cfg::D, R = Cfg::R, LPU = Cfg::LOADS_PER_UNIT;
     extern __shared__ __align__(16) uint8_t smem[];
     uint8_t *const a_stage = smem + Cfg::RING_BYTES;
@@ -295,9 +317,8 @@ gemm_skinny_stream_dma_kernel(const GemmArgs p, const int nblocks)
     const int Kb = p.K >> 1;
     const int nruns = (Kb + 127) >> 7;
     const int cnt = wave < nruns ? (nruns - wave + NW - 1) / NW : 0;  // this wave's runs: wave, wave + NW, ... (at most R)
-    const int G = gridDim.x;
-    const int my_blocks = ((int)blockIdx.x < nblocks) ? (nblocks - (int)blockIdx.x + G - 1) / G : 0;
-    const int units = my_blocks * cnt;  // (block, run) pairs of this wave, block-major
+    // (set after A's loads are on their way: the number of blocks takes a division)
+    int G, my_blocks, units;
 
     const int row8 = lane >> 3, pos = lane & 7;
     uint32_t piece_off[2];
@@ -317,7 +338,7 @@ gemm_skinny_stream_dma_kernel(const GemmArgs p, const int nblocks)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const uint32_t dst = ring_lds + slot * Cfg::UNIT_BYTES + (2 * j + h) * 1024;
-                const uint32_t goff = (uint32_t)min(n0 + j * 16 + 8 * h + row8, p.N - 1) * (uint32_t)Kb + min((uint32_t)run * 128u + piece_off[h], last16);
+                const uint32_t goff = row_bytes24(min(n0 + j * 16 + 8 * h + row8, p.N - 1), Kb) + min((uint32_t)run * 128u + piece_off[h], last16);
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(dst), "v"(goff), "s"(p.B) : "memory", "m0");
             }
         ++ld_u;
@@ -326,6 +347,9 @@ gemm_skinny_stream_dma_kernel(const GemmArgs p, const int nblocks)
 
     // ---- A first (it comes from the L2s and is needed by every block), then the ring ----
     const uint32_t a_lds = __builtin_amdgcn_readfirstlane(lds0 + Cfg::RING_BYTES + wave * R * FM * 2048);
+    // (issued the other way round -- B first, its requests out before A's pass through the L1 --
+    // the kernel is 10-15 % slower with B from HBM: every wave then waits for all of its loads
+    // before it can widen A)
 #pragma unroll
     for (int q = 0; q < R; ++q)
         if (q < cnt) {
@@ -334,10 +358,19 @@ gemm_skinny_stream_dma_kernel(const GemmArgs p, const int nblocks)
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const uint32_t dst = a_lds + (q * FM + i) * 2048 + h * 1024;
-                    const uint32_t goff = (uint32_t)min(i * 16 + 8 * h + row8, p.M - 1) * (uint32_t)Kb + min((uint32_t)(wave + q * NW) * 128u + piece_off[h], last16);
+                    const uint32_t goff = row_bytes24(min(i * 16 + 8 * h + row8, p.M - 1), Kb) + min((uint32_t)(wave + q * NW) * 128u + piece_off[h], last16);
                     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(goff), "s"(p.A) : "memory", "m0");
                 }
         }
+    {
+        // (the asm keeps the compiler from starting on the division before A's loads above)
+        int grid = out_and_grid >> 8;
+        asm volatile("" : "+s"(grid));
+        G = grid;
+        // one block per workgroup whenever the device holds them all at once: no division then
+        my_blocks = (int)blockIdx.x >= nblocks ? 0 : (G >= nblocks ? 1 : (nblocks - (int)blockIdx.x + G - 1) / G);
+        units = my_blocks * cnt;  // (block, run) pairs of this wave, block-major
+    }
     const int ahead = min(D, units);
     for (int d = 0; d < ahead; ++d) issue_unit();
 

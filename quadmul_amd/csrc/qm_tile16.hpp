@@ -233,10 +233,21 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         const int gsz = min(rows - first_m, group_m);
         const int tm_a = __builtin_amdgcn_readfirstlane(first_m + (pid % width) % gsz);
         const int tn_a = __builtin_amdgcn_readfirstlane((pid % width) / gsz);
-        // ragged tiles: the right column top to bottom (if N is ragged), then the bottom row
-        const int e = item - nwhole, right = tiles_n > full_n ? tiles_m : 0;
-        const int tm_b = e < right ? e : full_m, tn_b = e < right ? full_n : e - right;
+        // Ragged tiles: the right column top to bottom (if N is ragged) and the bottom row left to
+        // right, merged into one list in proportion (position q of nr holds right-column tile
+        // floor(q right / nr) where that quotient steps, a bottom-row tile otherwise), and the
+        // ragged items of one XCD (item % 8) take neighbouring positions of it, XCD 0 the head.
+        // An XCD's ragged tiles then lie beside the whole tiles it runs last -- the whole tiles
+        // are numbered top to bottom in the same XCD order -- and share panels with them and
+        // with each other in its L2, instead of every ragged tile fetching two panels of its own.
         const bool ragged = nwhole != 0 && item >= nwhole;
+        const int nr = max(nitems - nwhole, 1), right = tiles_n > full_n ? tiles_m : 0;
+        const int e8 = max(item - nwhole, 0) + (nwhole & 7), x8 = e8 & 7, s8 = nwhole & 7;
+        // positions before this XCD's: ragged items on lower XCDs, F(t) = integers in [0, t) with residue < x8
+        const int f_hi = ((s8 + nr) >> 3) * x8 + min((s8 + nr) & 7, x8), f_lo = min(s8, x8);
+        const int q = __builtin_amdgcn_readfirstlane(min(f_hi - f_lo + (e8 >> 3) - (x8 < s8 ? 1 : 0), nr - 1));
+        const int r0 = __builtin_amdgcn_readfirstlane(q * right / nr), r1 = __builtin_amdgcn_readfirstlane((q + 1) * right / nr);
+        const int tm_b = r1 > r0 ? r0 : full_m, tn_b = r1 > r0 ? full_n : q - r0;
         m0 = (ragged ? tm_b : tm_a) * BM;
         n0 = (ragged ? tn_b : tn_a) * BN;
         kt0 = __builtin_amdgcn_readfirstlane(min(ks * kps, kt_all - 1));

@@ -156,15 +156,21 @@ def test_selection_rules():
     assert name(4096, 4096, 96) == "generic"            # a single short K-step: nothing for the pipelined kernel to overlap it with
     # up to 64 rows: the wave-level split-K kernels; 3..16 rows stream their operands global ->
     # LDS, with a persistent grid and A resident in registers ("p") while the waves hold all of
-    # K, the plain form ("d") beyond
-    assert name(16, 4096, 4096) == "p1x1_w8_r2k2" and name(64, 4096, 4096) == "d4x1_w8_r1"
+    # K, the plain form ("d") beyond; from 33 rows the "d" form's grid walks over blocks of 32 rows
+    assert name(16, 4096, 4096) == "p1x1_w8_r2k2" and name(64, 4096, 4096) == "d2x2_w8_r1"
     assert name(1, 4096, 4096) == "v1x1_w4_u8" and name(1, 11008, 2048) == "v1x1_w8_u4" and name(2, 5120, 5120) == "v2x1_w16_u2"   # dot-product kernel
     assert name(1, 4096, 8192) == "v1x1_w16_u2" and name(2, 4096, 4096) == "v2x1_w8_u4"
     assert name(9, 28672, 14336) == "d1x1_w16_r1" and name(9, 11008, 8192) == "p1x1_w16_r2k2" and name(12, 2048, 2048) == "d1x1_w16_r1"
     assert name(3, 28672, 2048) == "p1x1_w8_r2k2" and name(16, 4096, 8192) == "d1x1_w16_r1"
     assert name(32, 11008, 4096) == "p2x1_w8_r2k2" and name(24, 4096, 2048) == "p2x1_w16_r2k1"
-    assert name(24, 4096, 8192) == "d2x1_w16_r1" and name(32, 28672, 8192) == "s2x1_w16_u2"
-    assert name(40, 4096, 14336) == "d4x1_w8_r1" and name(64, 11008, 4096) == "q64x64_w2x2_s8o2"
+    assert name(24, 4096, 8192) == "d2x1_w16_r1" and name(32, 28672, 8192) == "d2x2_w8_r1" and name(20, 2048, 8192) == "d1x1_w16_r1"
+    assert name(40, 4096, 14336) == "d2x2_w8_r1" and name(64, 11008, 4096) == "d2x2_w8_r1" and name(64, 2048, 4096) == "d2x1_w16_r1"
+    assert name(64, 16384, 4096) == "q64x64_w2x2_s8o2"
+    # a few hundred rows on few columns: the same 32 x 32 blocks, up to about three rounds of workgroups
+    assert name(128, 4096, 8192) == "d2x2_w8_r1" and name(192, 4096, 4096) == "d2x2_w8_r1" and name(96, 11008, 4096) == "d2x2_w8_r1"
+    assert name(128, 8192, 4096).startswith("q") and name(256, 4096, 4096).startswith("q") and name(128, 4096, 28672).startswith("q")
+    d22 = qm.config_id("d2x2_w8_r1")
+    assert qm.config_supports(d22, 1000, 4096, 4096) and not qm.config_supports(qm.config_id("p2x1_w8_r2k2"), 33, 4096, 4096)
     # a persistent "p" configuration only takes the K its waves hold in registers
     pk = qm.config_id("p1x1_w8_r2k2")
     assert qm.config_supports(pk, 16, 4096, 4096) and not qm.config_supports(pk, 16, 4096, 4096 + 32) and not qm.config_supports(pk, 17, 4096, 4096)
@@ -232,3 +238,65 @@ def test_w4a4_linear_argument_checks():
                 lambda: W4A4Linear(wq, ws, torch.zeros(7)), lambda: W4A4Linear(wq, ws, None, torch.float32)):
         with pytest.raises(qm.QuadmulError):
             bad()
+
+
+# --------------------------------------------------------------------------
+# Committed measurements must describe the kernels the library chooses today: a table row
+# retuned after the last profile / benchmark run fails here instead of leaving a stale figure.
+# --------------------------------------------------------------------------
+def _bench_module():
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("qm_bench_for_tests", os.path.join(ROOT, "bench.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_every_profile_summary_is_of_the_configuration_the_library_chooses():
+    bench = _bench_module()
+    profs = bench.profile_summaries()
+    assert profs, "no rocprofv3 summaries under profiles/"
+    for name, prof in profs.items():
+        m, n, k = prof["shape"]
+        scaled = name.endswith("_scaled_f16")
+        chosen = qm.config_name(qm.select_config_ex(m, n, k, scaled=scaled) & 0xFFFF)
+        assert prof["config"] == chosen, f"{prof['path']} profiled {prof['config']}, the library now chooses {chosen} for {m}x{n}x{k}"
+        # the file is named for the kernel, the configuration and the workload it covers
+        assert os.path.basename(prof["path"]).endswith(f"{prof['config']}__{name}.md"), prof["path"]
+        total = prof["traffic"]
+        assert 0.9 * bench.algorithmic_bytes(m, n, k) * (0.5 if scaled else 1.0) <= total <= 4 * bench.algorithmic_bytes(m, n, k), prof["path"]
+
+
+def test_bench_reads_traffic_from_the_summaries_for_every_workload_of_the_contract():
+    bench = _bench_module()
+    for name, (_, m, n, k, bound) in bench.WORKLOADS.items():
+        chosen = qm.config_name(qm.select_config(m, n, k) & 0xFFFF)
+        traffic, source = bench.profiled_traffic(name, m, n, k, chosen)
+        assert traffic is not None, f"{name}: {source}"
+        assert source.endswith(".md)") and f"__{name}.md" in source
+        if bound == "hbm":   # the HBM-fed figure these entries quote has a summary of its own
+            traffic_rot, source_rot = bench.profiled_traffic(name + "_rotating_b", m, n, k, chosen)
+            assert traffic_rot is not None, f"{name}_rotating_b: {source_rot}"
+    # a summary of another configuration is not used
+    t, why = bench.profiled_traffic("square8192", 8192, 8192, 8192, "q128x128_w2x2_s9o1")
+    assert t is None and "not used" in why
+
+
+def test_benchmark_table_rows_name_the_kernels_the_library_chooses():
+    path = os.path.join(ROOT, "benchmarks", "mi355x.md")
+    rows = [l for l in open(path).read().splitlines() if re.match(r"^\| \d+ \| \d+ \| \d+ \|", l)]
+    from quadmul_amd.autotune import REFERENCE_SHAPES
+
+    seen = set()
+    for l in rows:
+        cells = [c.strip() for c in l.strip("|").split("|")]
+        m, n, k = int(cells[0]), int(cells[1]), int(cells[2])
+        kernel = cells[-1]
+        if (m, n, k) in seen:     # (the second table, timed through the bare seven-argument entry point)
+            chosen = qm.config_name(qm.select_config_ex(m, n, k, workspace=False) & 0xFFFF)
+        else:
+            chosen = qm.config_name(qm.select_config(m, n, k) & 0xFFFF)
+        seen.add((m, n, k))
+        assert kernel == chosen, f"benchmarks/mi355x.md row {m}x{n}x{k} names {kernel}, the library chooses {chosen}: regenerate the table"
+    assert seen == set(REFERENCE_SHAPES), "the table must cover the reference's 42 shapes (kernel.cu:343-384)"

@@ -432,7 +432,7 @@ def test_random_shapes_through_the_automatic_choice():
         # in the workspace (which quadmul.gemm provides)
         if name == "generic" and m * n * ((k + 127) // 128 * 128) >= 2 ** 27 and k <= 131000:
             assert qm.workspace_bytes(m, n, k) > 0, (m, n, k)
-    assert {"g", "s", "q", "q+split"} <= seen, seen
+    assert {"g", "d", "p", "q", "q+split"} <= seen, seen
 
 
 @pytest.mark.parametrize("shape", [(1, 4096, 4096), (2, 4100, 11008), (1, 50, 131040), (2, 33, 28672), (1, 4096, 96)],
@@ -676,11 +676,13 @@ def test_skinny_kernel_walking_over_column_blocks(oracle_mod, shape):
 
 
 @pytest.mark.parametrize("shape", [(16, 9000, 4096), (3, 8210, 1024 + 32), (30, 4100, 2048 + 96), (13, 5000, 8192), (16, 300, 14336 + 64),
-                                   (50, 4200, 4096 + 32), (7, 33, 32), (16, 16, 65536)],
+                                   (50, 4200, 4096 + 32), (7, 33, 32), (16, 16, 65536),
+                                   # several blocks of rows (the "d" form's grid walks over them), the last one ragged
+                                   (64, 4096, 4096), (100, 4200, 4096 + 32), (200, 1000, 2048 + 64), (129, 530, 8192), (33, 8300, 256)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_skinny_kernels_streaming_global_to_lds(oracle_mod, shape):
     """The skinny kernels whose operands go global -> LDS directly ("d": one workgroup per
-    column block, a ring of runs per wave refilled over a long K; "p": a persistent grid
+    block of rows and of columns, a ring of runs per wave refilled over a long K; "p": a persistent grid
     walking over more column blocks than the device holds workgroups, A resident in
     registers): ragged N, short last runs of K (K % 256 = 32, 64, 96), K from one run to 256
     runs per row.  Every such configuration that takes the shape, int32 and scaled output,
@@ -723,14 +725,15 @@ def test_every_config_on_random_shapes_against_the_generic_kernel():
     rng = np.random.default_rng(SEED_BASE + 77)
     names = qm.config_names()
     generic = names.index("generic")
-    skinny_m = [1, 2, 3, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64]
+    skinny_m = [1, 2, 3, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100, 129, 200]
     skinny_n = [1, 5, 16, 17, 100, 255, 256, 1000, 4096, 4100, 9000]
     skinny_k = [1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 32, 33, 64, 100, 127, 128, 129, 256, 300]
     tile_m = [1, 16, 63, 64, 65, 128, 200, 256, 257, 512, 700]
     tile_n = [8, 64, 100, 128, 256, 260, 512, 1000, 1300]
     tile_k = [1, 2, 3, 4, 5, 8, 12, 13, 16, 31, 32, 40, 64, 65]
     ran = {}
-    for _ in range(20000):
+    gen = torch.Generator(device=DEV)
+    for it in range(20000):
         cfg = int(rng.integers(len(names)))
         if cfg == generic:
             continue
@@ -740,13 +743,15 @@ def test_every_config_on_random_shapes_against_the_generic_kernel():
         k = 32 * int(rng.choice(tile_k if tile else skinny_k))
         if not qm.config_supports(cfg, m, n, k):
             continue
-        a = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=DEV)
-        b = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=DEV)
+        seed = SEED_BASE + 770000 + it   # of this case's operands: a failure can be replayed alone
+        gen.manual_seed(seed)
+        a = torch.randint(0, 256, (m, k // 2), dtype=torch.uint8, device=DEV, generator=gen)
+        b = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=DEV, generator=gen)
         want = poisoned_c(m, n, DEV)
         qm.gemm_cfg(a, b, want, m, n, k, generic)
         ksplit = int(rng.choice([1, 1, 2, 3])) if tile and k >= 256 else 1
         got = poisoned_c(m, n, DEV)
         qm.gemm_cfg(a, b, got, m, n, k, cfg | (ksplit << 24) if ksplit > 1 else cfg, workspace=True if rng.integers(2) else None)
-        assert torch.equal(want, got), (names[cfg], ksplit, m, n, k)
+        assert torch.equal(want, got), (names[cfg], ksplit, m, n, k, f"operand seed {seed}")
         ran[names[cfg]] = ran.get(names[cfg], 0) + 1
     assert len(ran) == len(names) - 1 and min(ran.values()) >= 10, ran
