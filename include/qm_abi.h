@@ -50,6 +50,22 @@ extern "C" {
  * with the same seven arguments in the same order plus a status.  Unlike the
  * reference, every shape with m,n >= 0 and even k >= 0 is computed (m or n == 0
  * is a no-op, k == 0 zero-fills C).
+ *
+ * Seven arguments leave no room for a workspace.  On every shape whose best schedule needs
+ * none -- 36 of the 42 shapes of the reference's table (kernel.cu:343-384), every BASELINE
+ * shape, K below one 128-nibble step -- this entry point runs exactly what qm_gemm_i4_ws
+ * runs.  It is slower than qm_gemm_i4_ws / qm_gemm_i4_static (measured, MI355X, both columns
+ * of benchmarks/mi355x.md's second table) in two cases:
+ *   - few output tiles and a long K, which those entry points split over several workgroups
+ *     per tile through the workspace: here the best unsplit configuration runs instead.
+ *     128 x 8192 x 28672: 51.8 us against 35.7 (1.45x); 256 x 8192 x 28672: 70.8 against
+ *     54.4 (1.30x); the other four such rows of the reference's table (512 x 8192 x 28672,
+ *     256 and 512 x 4096 x 14336, 128 x 10240 x 8192) within 10 %;
+ *   - K % 32 != 0, or A or B not 16-byte aligned: no 16-byte loads, the one-thread-per-element
+ *     kernel runs (2048 x 4096 x 4100: 3.3 ms, against 44 us on zero-padded copies in a
+ *     workspace).  Weight matrices of the reference's table all have K % 32 == 0.
+ * A caller that can lend device memory should bind qm_gemm_i4_ws; one that cannot allocate,
+ * qm_gemm_i4_static.
  */
 int qm_gemm_i4(const void *A, const void *B, void *C, int m, int n, int k, void *stream);
 

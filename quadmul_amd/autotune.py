@@ -159,19 +159,33 @@ def tune_shape(m: int, n: int, k: int, device, group_ms: Iterable[int], min_ms: 
     print(f"{m}x{n}x{k}: best {best['config']} gm={best['group_m']} ks={best['ksplit']} spread={best['spread']} {best['ms']*1e3:.1f} us "
           f"{best['tops']:.1f} TOPS ({100*best['tops']/INT8_PEAK_TOPS:.1f}% int8 peak) "
           f"{best['gbs']:.0f} GB/s ({100*best['gbs']/HBM_PEAK_GBS:.1f}% HBM)", flush=True)
-    return {"m": m, "n": n, "k": k, "best": best, "all": results}
+    out = {"m": m, "n": n, "k": k, "best": best, "all": results}
+    if best["ksplit"] > 1:
+        # The best choice splits K through a workspace.  Callers of the bare seven-argument
+        # entry point have none: their row gets a second choice, the best unsplit one.  (An
+        # unsplit launch runs the same with and without a workspace, so the times above hold;
+        # a K split whose partial sums meet in C through atomics was measured behind the best
+        # unsplit configuration on every shape of the reference's table.)
+        nows = next(r for r in results if r["ksplit"] == 1)
+        out["best_without_workspace"] = nows
+        print(f"    without a workspace: {nows['config']} gm={nows['group_m']} {nows['ms']*1e3:.1f} us", flush=True)
+    return out
 
 
 def emit_table(tuned: List[Dict], path: str) -> None:
     lines = [
         "// Per-shape kernel choice measured on MI355X: {M, N, K, \"config name\", group_m, ksplit,",
-        "// one item per workgroup}.",
+        "// one item per workgroup[, \"config name\" and group_m for calls without a workspace, on rows",
+        "// whose first choice splits K through one]}.",
         "// Written by quadmul_amd/autotune.py; shapes not listed use the cost model in",
         "// qm_select.hpp.  Counterpart of the reference's A40 table (configs.cu:19-689).",
     ]
     for t in tuned:
         b = t["best"]
-        lines.append(f"{{{t['m']}, {t['n']}, {t['k']}, \"{b['config']}\", {b['group_m']}, {b['ksplit']}, {b.get('spread', 0)}}},  // {b['ms']*1e3:.1f} us, {b['tops']:.0f} TOPS")
+        nows = t.get("best_without_workspace")
+        extra = f", \"{nows['config']}\", {nows['group_m']}" if nows else ""
+        note = f" ({nows['ms']*1e3:.1f} us without a workspace)" if nows else ""
+        lines.append(f"{{{t['m']}, {t['n']}, {t['k']}, \"{b['config']}\", {b['group_m']}, {b['ksplit']}, {b.get('spread', 0)}{extra}}},  // {b['ms']*1e3:.1f} us, {b['tops']:.0f} TOPS{note}")
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
 

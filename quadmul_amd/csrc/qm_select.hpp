@@ -107,6 +107,10 @@ struct TableEntry {
     const char *config;
     int group_m, ksplit;
     int spread;  // 1: one work item per workgroup instead of a persistent grid (pipelined kernel)
+    // rows whose choice splits K through a workspace: the measured choice for calls that have
+    // none (the bare seven-argument entry point), never split
+    const char *nows_config = nullptr;
+    int nows_group_m = 0;
 };
 static const TableEntry g_table[] = {
 #include "qm_tile_table.inc"
@@ -153,6 +157,15 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         if (n <= 2048) return pick("d2x1_w16_r1");
         if (n <= 12288) return pick("d2x2_w8_r1");
         if (n <= 16384 && config_supports(find_config("q64x64_w2x2_s8o2"), m, n, k, ptr_align)) return pick("q64x64_w2x2_s8o2");
+    }
+    if (k < 128) {
+        // A K of one short step (32, 64 or 96) is nothing for the pipelined kernel: it has no
+        // earlier step to overlap that one with.  The 32 x 32 blocks take any number of rows;
+        // one wave per workgroup when there are thousands of them (only one wave has a run of
+        // K to work on).  Measured: 2048 x 4096 x 96 13.0 us (eight waves: 27.7; the generic
+        // kernel: 114; on zero-padded copies in a workspace: 11.9), 8192 x 8192 x 96 66 us (875; 56).
+        const long long wgs = (long long)((m + 31) / 32) * ((n + 31) / 32);
+        return pick(wgs > 1024 ? "d2x2_w1_r1" : "d2x2_w8_r1");
     }
     if (m <= 256 && k <= 16384) {
         // The same 32 x 32 blocks on a few hundred rows (measured with B from HBM, M = 65 .. 256,
@@ -201,7 +214,9 @@ tiles:
             int t = 1;
             while (t < 4 && tiles * t * 2 <= 256 && (k / 128) / (t * 2) >= 48) t *= 2;
             if (t > 1) {
-                const double split_cost = (double)d.bm * d.bn / c.eff * ((kt + t - 1) / t) * 1.25 + 180000.0;
+                // (+ one 4-byte atomic per element and split at about 10 ps each, 0.6 units --
+                // measured: 512 x 8192 x 28672 in four splits 253 us, 170 of them the atomics)
+                const double split_cost = (double)d.bm * d.bn / c.eff * ((kt + t - 1) / t) * 1.25 + 180000.0 + 0.6 * (double)m * (double)n * t;
                 if (split_cost < cost) { cost = split_cost; ks = t; }
             }
         }
@@ -223,18 +238,25 @@ tiles:
 
 static Choice select_config(int m, int n, int k, int ptr_align, bool has_ws)
 {
-    static int resolved[sizeof(g_table) / sizeof(g_table[0])];
+    static int resolved[sizeof(g_table) / sizeof(g_table[0])], resolved_nows[sizeof(g_table) / sizeof(g_table[0])];
     static std::once_flag once;
     std::call_once(once, [] {
-        for (size_t i = 0; g_table[i].config; ++i) resolved[i] = find_config(g_table[i].config);
+        for (size_t i = 0; g_table[i].config; ++i) {
+            resolved[i] = find_config(g_table[i].config);
+            resolved_nows[i] = g_table[i].nows_config ? find_config(g_table[i].nows_config) : -1;
+        }
     });
     for (size_t i = 0; g_table[i].config; ++i)
         if (g_table[i].m == m && g_table[i].n == n && g_table[i].k == k && resolved[i] >= 0 &&
             config_supports(resolved[i], m, n, k, ptr_align)) {
             // The table's K splits were measured through the workspace (partial tiles, then the
-            // kernel that adds them up).  Without one the partial sums would meet in C through
-            // atomics, which is priced differently: the cost model decides.
-            if (g_table[i].ksplit > 1 && !has_ws) break;
+            // kernel that adds them up).  Without one the row's second choice runs, measured
+            // without a workspace; where a row has none, the cost model decides.
+            if (g_table[i].ksplit > 1 && !has_ws) {
+                if (resolved_nows[i] >= 0 && config_supports(resolved_nows[i], m, n, k, ptr_align))
+                    return {resolved_nows[i], g_table[i].nows_group_m > 0 ? g_table[i].nows_group_m : 4, 1, 0};
+                break;
+            }
             return {resolved[i], g_table[i].group_m, g_table[i].ksplit > 0 ? g_table[i].ksplit : 1, g_table[i].spread};
         }
     return heuristic(m, n, k, ptr_align, has_ws);

@@ -351,7 +351,7 @@ gemm_dot_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int M, con
     p.out = out;
     p.ldc = ldc;
     constexpr int MR = Cfg::MR, FN = Cfg::FN, NW = Cfg::NW, U = Cfg::U;
-    __shared__ int32_t red[MR][FN * 16];  // the sum over the waves
+    __shared__ int32_t red[NW][MR][FN * 16];  // every wave's sums, added up after one barrier (nothing to clear, no barrier in front of the loads)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n0 = blockIdx.x * Cfg::BN;
@@ -374,9 +374,6 @@ gemm_dot_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int M, con
     for (int i = 0; i < MR; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j][0] = acc[i][j][1] = 0;
-    for (int idx = tid; idx < MR * FN * 16; idx += Cfg::THREADS) (&red[0][0])[idx] = 0;
-    __syncthreads();
-
     for (int c0 = wave * U; c0 < nchunks; c0 += NW * U) {
         v4i bq[U / 2][FN][2], aq[U / 2][MR];
 #pragma unroll
@@ -406,7 +403,7 @@ gemm_dot_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int M, con
 
     // the eight lanes of a row hold the eight 32-nibble pieces of a pair of chunks: add them
     // up (within the quads, then the two quads through the mirror image of the eight), then
-    // the waves' sums in the LDS
+    // the waves' sums through the LDS
 #pragma unroll
     for (int i = 0; i < MR; ++i)
 #pragma unroll
@@ -417,13 +414,15 @@ gemm_dot_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int M, con
                 v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
                 v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
                 v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);  // row_half_mirror: lane i <-> 7 - i
-                if (ld_ch == 0) __hip_atomic_fetch_add(&red[i][j * 16 + 8 * h + ld_row], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (ld_ch == 0) red[wave][i][j * 16 + 8 * h + ld_row] = v;
             }
     __syncthreads();
     for (int idx = tid; idx < MR * FN * 16; idx += Cfg::THREADS) {
         const int m = idx / (FN * 16), n = n0 + idx % (FN * 16);
         if (m < p.M && n < p.N) {
-            const int32_t s = (&red[0][0])[idx];
+            int32_t s = 0;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) s += (&red[w][0][0])[idx];
             const size_t at = (size_t)m * c_stride(p) + n;
             if (p.out == OUT_I32) p.C[at] = s;
             else reinterpret_cast<uint16_t *>(p.C)[at] = round16(scaled(s, scale_at(p.row_scale, m, p.M), scale_at(p.col_scale, n, p.N)), p.out);

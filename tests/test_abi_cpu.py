@@ -153,7 +153,9 @@ def test_selection_rules():
     assert name(8192, 8192, 8192).startswith("q")   # pipelined 16x16x64 kernel: K % 128 == 0
     assert name(4096, 4096, 4096).startswith("q")
     assert name(4096, 4096, 4096 + 32).startswith("q")  # K % 32 == 0: the pipelined kernel with a short last K-step
-    assert name(4096, 4096, 96) == "generic"            # a single short K-step: nothing for the pipelined kernel to overlap it with
+    # a single short K-step: nothing for the pipelined kernel to overlap it with; 32 x 32 blocks of the wave-level kernel
+    assert name(4096, 4096, 96) == "d2x2_w1_r1" and name(300, 300, 64) == "d2x2_w8_r1" and name(4096, 4096, 128).startswith("q")
+    assert qm.workspace_bytes(4096, 4096, 96) == 0
     # up to 64 rows: the wave-level split-K kernels; 3..16 rows stream their operands global ->
     # LDS, with a persistent grid and A resident in registers ("p") while the waves hold all of
     # K, the plain form ("d") beyond; from 33 rows the "d" form's grid walks over blocks of 32 rows
@@ -180,13 +182,13 @@ def test_selection_rules():
     assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
     assert (qm.select_config(8192, 8192, 8192) >> 24) & 0x3F == 1
     # ... which the table's rows were measured with: without a workspace (the plain 7-argument
-    # call) the cost model decides, and keeps a split only where it is priced below none
-    for (m, n, k) in [(128, 10240, 8192), (256, 4096, 14336), (512, 8192, 28672), (128, 8192, 28672)]:
+    # call) such a row's second, unsplit choice runs (measured without one); the cost model
+    # for untabled shapes prices the atomics of a split without a workspace and keeps none here
+    for (m, n, k) in [(128, 10240, 8192), (256, 4096, 14336), (512, 8192, 28672), (128, 8192, 28672), (384, 8192, 28672)]:
         with_ws, without = qm.select_config_ex(m, n, k, workspace=True), qm.select_config_ex(m, n, k, workspace=False)
         assert (with_ws >> 24) & 0x3F > 1 and with_ws == qm.select_config(m, n, k)
-        assert qm.config_name(without & 0xFFFF).startswith("q")
-        if k <= 8192:
-            assert (without >> 24) & 0x3F == 1, (m, n, k)   # atomics lose at this K (measured)
+        assert qm.config_name(without & 0xFFFF).startswith(("q", "d2x2")) and (without >> 24) & 0x3F == 1, (m, n, k)
+    assert qm.config_name(qm.select_config_ex(512, 8192, 28672, workspace=False) & 0xFFFF) == "q128x128_w2x2_s9o1"
     # scaled output, no workspace, long K with a short last K-step: a pipelined configuration
     # that has the output form, never the generic kernel
     for (m, n, k) in [(256, 256, 28704), (128, 8192, 28672 + 32), (512, 4096, 14336 + 96)]:

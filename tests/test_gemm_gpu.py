@@ -463,9 +463,10 @@ def test_dot_product_kernel_one_and_two_rows(oracle_mod, shape):
                                    (2100, 4200, 96), (1500, 1500, 64), (4096, 4096, 32)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_k_padded_through_the_workspace(shape):
-    """Large shapes whose K is not a multiple of 32 or is less than one K-step, and unaligned
-    operands: with a workspace the operands are copied with zero-padded rows and the
-    pipelined kernel runs; without one the generic kernel does.  (K % 32 == 0, first case: no copies, a short last K-step.)  Same
+    """Large shapes whose K is not a multiple of 32, and unaligned operands: with a workspace
+    the operands are copied with zero-padded rows and the pipelined kernel runs; without one
+    the generic kernel does.  (K % 32 == 0, first case: no copies, a short last K-step; a K of
+    less than one K-step: no copies either, 32 x 32 blocks of the wave-level kernel.)  Same
     result, against an exact fp32 matmul."""
     import quadmul
 
@@ -475,8 +476,10 @@ def test_k_padded_through_the_workspace(shape):
     want = fp32_matmul_on_gpu(a, b)
     ap, bp = pack_cpu(a), pack_cpu(b)
     a_d, b_d = ap.to(DEV), bp.to(DEV)
-    if k % 32 or k < 128:   # (less than one whole K-step: nothing for a short last step to follow)
+    if k % 32:
         assert qm.workspace_bytes(m, n, k) >= (m + n) * ((k + 127) // 128 * 64)
+    elif k < 128:   # (less than one whole K-step: nothing for a short last step to follow)
+        assert qm.workspace_bytes(m, n, k) == 0 and qm.config_name(qm.select_config(m, n, k) & 0xFFFF).startswith("d2x2")
     else:   # K % 32 == 0: the pipelined kernel runs it as it is, with a short last K-step
         assert qm.workspace_bytes(m, n, k) == 0 and qm.config_name(qm.select_config(m, n, k) & 0xFFFF).startswith("q")
     for fn in (lambda c: quadmul.gemm(a_d, b_d, c, m, n, k), lambda c: qm.gemm(a_d, b_d, c, m, n, k),
