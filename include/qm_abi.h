@@ -211,6 +211,17 @@ int qm_quantize_pack_i4(const void *x, int in_dtype, void *dst_packed, float *sc
  */
 int qm_init(void);
 
+/*
+ * Testing aid, not for production callers.  Operands of 2 GiB and more are cut by the library
+ * into blocks its kernels' 32-bit row offsets reach: blocks of rows of A, and blocks of rows
+ * of B, which are blocks of columns of C written through a row stride.  This call lowers that
+ * limit (bytes; <= 0 restores 2^31 - 1) so that the block paths can be driven on small
+ * shapes; it returns the previous limit.  Process-wide, not synchronised with calls in
+ * flight on other threads.  No counterpart in the reference (its kernels take no operand
+ * beyond their table's shapes, kernel.cu:340-385).
+ */
+long long qm_debug_set_operand_limit(long long bytes);
+
 /* Diagnostics.  qm_version names the compiler the library was built with: the kernels
  * manage matrix-core hazards by hand, so a result is validated for that compiler. */
 const char *qm_status_string(int status);

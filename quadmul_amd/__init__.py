@@ -37,6 +37,7 @@ ABI_SYMBOLS = (
     "qm_gemm_i4", "qm_gemm_i4_cfg", "qm_gemm_i4_scaled", "qm_gemm_i4_scaled_cfg", "qm_config_has_scaled",
     "qm_gemm_i4_ws", "qm_gemm_i4_static", "qm_gemm_i4_scaled_ws", "qm_gemm_workspace_bytes", "qm_quantize_pack_i4", "qm_select_config", "qm_select_config_ex", "qm_num_configs", "qm_config_name",
     "qm_config_supports", "qm_pack_i4", "qm_unpack_i4", "qm_status_string", "qm_last_hip_error", "qm_version", "qm_init",
+    "qm_debug_set_operand_limit",
 )
 
 
@@ -101,6 +102,8 @@ def library() -> ctypes.CDLL:
     lib.qm_init.restype = ci
     lib.qm_version.argtypes = []
     lib.qm_version.restype = ctypes.c_char_p
+    lib.qm_debug_set_operand_limit.argtypes = [ctypes.c_longlong]
+    lib.qm_debug_set_operand_limit.restype = ctypes.c_longlong
     _lib = lib
     return lib
 
@@ -348,6 +351,12 @@ def select_config_ex(m: int, n: int, k: int, ptr_align: int = 256, workspace: bo
 
 def config_supports(cfg: int, m: int, n: int, k: int, ptr_align: int = 256) -> bool:
     return bool(library().qm_config_supports(cfg, m, n, k, ptr_align))
+
+
+def debug_set_operand_limit(nbytes: int) -> int:
+    """Testing aid: operands of ``nbytes`` or more are cut into blocks (0 restores 2 GiB - 1);
+    returns the previous limit.  See ``qm_debug_set_operand_limit`` in include/qm_abi.h."""
+    return int(library().qm_debug_set_operand_limit(nbytes))
 
 
 def version() -> str:

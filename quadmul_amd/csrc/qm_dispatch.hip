@@ -248,6 +248,12 @@ static hipError_t launch_split_with_workspace(GemmArgs p, const Choice &ch, void
     return hipGetLastError();
 }
 
+// Operands of this many bytes or more are cut into blocks (below).  2^31 - 1 in production: what
+// the kernels' 32-bit row offsets reach.  qm_debug_set_operand_limit lowers it so that tests
+// can drive the block paths -- C written through a row stride, blocks of rows then of columns --
+// on small shapes.
+static std::atomic<long long> g_operand_limit{0x7fffffffLL};
+
 // An A of 2 GiB or more is beyond the 32-bit row offsets of the fast kernels; its row blocks
 // are independent (block r0.. of A gives rows r0.. of C), so the call is cut into blocks
 // of rows that fit, one after the other on the stream (they share the workspace).  Returns
@@ -257,9 +263,9 @@ static int row_block_for_large_a(int m, int n, int k, int ptr_align)
 {
     (void)n;
     if (k < 32 || k % 32 != 0 || k > QM_MAX_K_X16 || ptr_align < 16) return 0;
-    const long long kb = k / 2;
-    if ((long long)m * kb < 0x7fffffffLL) return 0;
-    const long long rows = ((0x7fffffffLL - 1) / kb) & ~255LL;
+    const long long kb = k / 2, limit = g_operand_limit.load(std::memory_order_relaxed);
+    if ((long long)m * kb < limit) return 0;
+    const long long rows = ((limit - 1) / kb) & ~255LL;
     return rows >= 256 ? (int)rows : 0;
 }
 
@@ -268,9 +274,9 @@ static int row_block_for_large_a(int m, int n, int k, int ptr_align)
 static int col_block_for_large_b(int m, int n, int k, int ptr_align)
 {
     if (k < 32 || k % 32 != 0 || k > QM_MAX_K_X16 || ptr_align < 16) return 0;
-    const long long kb = k / 2;
-    if ((long long)n * kb < 0x7fffffffLL || (long long)m * kb >= 0x7fffffffLL) return 0;
-    const long long cols = ((0x7fffffffLL - 1) / kb) & ~255LL;
+    const long long kb = k / 2, limit = g_operand_limit.load(std::memory_order_relaxed);
+    if ((long long)n * kb < limit || (long long)m * kb >= limit) return 0;
+    const long long cols = ((limit - 1) / kb) & ~255LL;
     return cols >= 256 ? (int)cols : 0;
 }
 
@@ -584,6 +590,12 @@ QM_EXPORT const char *qm_status_string(int status)
 }
 
 QM_EXPORT int qm_last_hip_error(void) { return g_last_hip_error; }
+
+QM_EXPORT long long qm_debug_set_operand_limit(long long bytes)
+{
+    const long long full = 0x7fffffffLL;
+    return g_operand_limit.exchange(bytes <= 0 || bytes > full ? full : bytes, std::memory_order_relaxed);
+}
 
 #ifndef QM_COMPILER_VERSION
 #define QM_COMPILER_VERSION "unknown compiler"
