@@ -600,4 +600,4 @@ QM_EXPORT long long qm_debug_set_operand_limit(long long bytes)
 #ifndef QM_COMPILER_VERSION
 #define QM_COMPILER_VERSION "unknown compiler"
 #endif
-QM_EXPORT const char *qm_version(void) { return "quadmul-amd 0.2 (gfx950; built with " QM_COMPILER_VERSION ")"; }
+QM_EXPORT const char *qm_version(void) { return "quadmul-amd 0.3 (gfx950; built with " QM_COMPILER_VERSION ")"; }

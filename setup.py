@@ -28,11 +28,12 @@ class BuildNative(build_ext):
     def run(self):
         from quadmul_amd import build as qbuild
 
-        libs = [qbuild.LIB_PATH, qbuild.PROBE_PATH]
+        # (the measurement probes of bench.py, libqm_probe.so, stay in the tree: a user of the
+        # library has no use for them)
+        libs = [qbuild.LIB_PATH]
         reuse = os.environ.get("QM_REUSE_BUILD") == "1" and all(os.path.exists(p) for p in libs + [qbuild.ext_path()])
         if not reuse:
             qbuild.build_lib(jobs=int(os.environ.get("MAX_JOBS", "8")))
-            qbuild.build_probe()
             qbuild.build_ext()
         # the extension module: looks for libqm_hip.so in quadmul_amd/lib beside it ($ORIGIN rpath)
         dst = self.get_ext_fullpath("quadmul")
@@ -48,16 +49,16 @@ class BuildNative(build_ext):
     def get_outputs(self):
         outs = [self.get_ext_fullpath("quadmul")]
         if not self.inplace:
-            outs += [os.path.join(self.build_lib, "quadmul_amd", "lib", n) for n in ("libqm_hip.so", "libqm_probe.so")]
+            outs += [os.path.join(self.build_lib, "quadmul_amd", "lib", "libqm_hip.so")]
         return outs
 
 
 setup(
     name="quadmul",
-    version="0.2",
+    version="0.3",
     description="Packed int4 x int4 -> int32 GEMM for AMD MI355X (gfx950): drop-in for quadmul.gemm",
     packages=["quadmul_amd"],
-    package_data={"quadmul_amd": ["csrc/*", "lib/*.so"]},
+    package_data={"quadmul_amd": ["csrc/*", "lib/libqm_hip.so"]},
     ext_modules=[Extension("quadmul", sources=[])],   # built by quadmul_amd.build, not by setuptools
     cmdclass={"build_ext": BuildNative},
     python_requires=">=3.9",

@@ -24,6 +24,7 @@ def test_pip_install_into_a_prefix_and_import_from_outside(tmp_path):
     names = os.listdir(target)
     assert any(n.startswith("quadmul.") and n.endswith(".so") for n in names), names
     assert os.path.exists(target / "quadmul_amd" / "lib" / "libqm_hip.so")
+    assert not os.path.exists(target / "quadmul_amd" / "lib" / "libqm_probe.so")   # bench.py's instruments stay in the tree
     code = ("import sys, os; assert not any(os.path.abspath(p or '.') == %r for p in sys.path); "
             "import quadmul, quadmul_amd; "
             "assert quadmul.__file__.startswith(%r) and quadmul_amd.__file__.startswith(%r); "
