@@ -52,15 +52,14 @@ extern "C" {
  * is a no-op, k == 0 zero-fills C).
  *
  * Seven arguments leave no room for a workspace.  On every shape whose best schedule needs
- * none -- 36 of the 42 shapes of the reference's table (kernel.cu:343-384), every BASELINE
+ * none -- 40 of the 42 shapes of the reference's table (kernel.cu:343-384), every BASELINE
  * shape, K below one 128-nibble step -- this entry point runs exactly what qm_gemm_i4_ws
  * runs.  It is slower than qm_gemm_i4_ws / qm_gemm_i4_static (measured, MI355X, both columns
  * of benchmarks/mi355x.md's second table) in two cases:
  *   - few output tiles and a long K, which those entry points split over several workgroups
  *     per tile through the workspace: here the best unsplit configuration runs instead.
- *     128 x 8192 x 28672: 51.8 us against 35.7 (1.45x); 256 x 8192 x 28672: 70.8 against
- *     54.4 (1.30x); the other four such rows of the reference's table (512 x 8192 x 28672,
- *     256 and 512 x 4096 x 14336, 128 x 10240 x 8192) within 10 %;
+ *     256 x 8192 x 28672: 70.7 us against 54.9 (1.29x); 512 x 8192 x 28672: 95.9 against
+ *     92.5 (1.04x); no other shape of the reference's table splits K;
  *   - K % 32 != 0, or A or B not 16-byte aligned: no 16-byte loads, the one-thread-per-element
  *     kernel runs (2048 x 4096 x 4100: 3.3 ms, against 44 us on zero-padded copies in a
  *     workspace).  Weight matrices of the reference's table all have K % 32 == 0.

@@ -167,6 +167,22 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         const long long wgs = (long long)((m + 31) / 32) * ((n + 31) / 32);
         return pick(wgs > 1024 ? "d2x2_w1_r1" : "d2x2_w8_r1");
     }
+    if (m <= 512 && k >= 2048 && k <= 32768) {
+        // A few hundred rows on few columns: blocks of 64 x 64 or 64 x 32 of the same kernel, one
+        // workgroup per CU, when that makes one round of workgroups that fills most of the
+        // device -- a workgroup pulls (rows + columns) x K / 2 bytes through its L1 for rows x
+        // columns x K multiply-adds, so the larger block moves half as much per product.
+        // Measured with B from HBM, M = 96 .. 512, N = 2048 .. 8192, K = 4096 .. 28672, against
+        // the tiles and the 32 x 32 blocks: 128 x 8192 x 8192 15.4 us (64 x 64 tiles: 19.1),
+        // 256 x 4096 x 8192 14.5 (18.8), 512 x 2048 x 4096 8.7 (11.3), 128 x 4096 x 8192 9.6 on
+        // 64 x 32 (32 x 32: 11.1).  Two rounds lose to the tiles, except on a long K without a
+        // workspace to split it through.
+        const long long r64 = (m + 63) / 64, c64 = (n + 63) / 64, c32 = (n + 31) / 32, r32 = (m + 31) / 32;
+        if (r64 * c64 >= 140 && r64 * c64 <= 256) return pick("d4x4_w8_r1");
+        if (!has_ws && k >= 8192 && r64 * c64 > 256 && r64 * c64 <= 512) return pick("d4x4_w8_r1");
+        if (r64 * c32 >= 140 && r64 * c32 <= 256) return pick("d4x2_w8_r1");
+        if (r32 * c64 >= 140 && r32 * c64 <= 256) return pick("d2x4_w8_r1");
+    }
     if (m <= 256 && k <= 16384) {
         // The same 32 x 32 blocks on a few hundred rows (measured with B from HBM, M = 65 .. 256,
         // N = 2048 .. 11008, K = 2048 .. 8192): ahead of the tiles -- no ring to fill, one

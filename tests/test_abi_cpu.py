@@ -118,10 +118,11 @@ def test_workspace_sizes():
     assert qm.workspace_bytes(200, 300, 4096, q128) == 0                       # no split asked for
     assert qm.workspace_bytes(16, 300, 4096, qm.config_id("s1x1_w8_u4") | (4 << 24)) == 0
     assert qm.workspace_bytes(8192, 8192, 8192) == 0                           # plenty of tiles
-    code = qm.select_config(128, 8192, 28672)
+    code = qm.select_config(256, 8192, 28672)
     assert (code >> 24) & 0x3F > 1
-    assert qm.workspace_bytes(128, 8192, 28672) == qm.workspace_bytes(128, 8192, 28672, code) > 0
-    assert qm.workspace_bytes(128, 8192, 28672, scaled=True) > 0
+    assert qm.workspace_bytes(256, 8192, 28672) == qm.workspace_bytes(256, 8192, 28672, code) > 0
+    assert qm.workspace_bytes(256, 8192, 28672, scaled=True) > 0
+    assert qm.workspace_bytes(128, 8192, 28672) == 0                          # one round of 64 x 64 blocks of the wave-level kernel
     assert qm.workspace_bytes(0, 8192, 28672) == 0 and qm.workspace_bytes(128, 8192, 3) == 0
     # large shapes with K % 32 != 0 (or unaligned operands): room for copies of A and B with rows
     # padded to whole K-steps
@@ -169,8 +170,11 @@ def test_selection_rules():
     assert name(40, 4096, 14336) == "d2x2_w8_r1" and name(64, 11008, 4096) == "d2x2_w8_r1" and name(64, 2048, 4096) == "d2x1_w16_r1"
     assert name(64, 16384, 4096) == "q64x64_w2x2_s8o2"
     # a few hundred rows on few columns: the same 32 x 32 blocks, up to about three rounds of workgroups
-    assert name(128, 4096, 8192) == "d2x2_w8_r1" and name(192, 4096, 4096) == "d2x2_w8_r1" and name(96, 11008, 4096) == "d2x2_w8_r1"
-    assert name(128, 8192, 4096).startswith("q") and name(256, 4096, 4096).startswith("q") and name(128, 4096, 28672).startswith("q")
+    assert name(128, 2048, 8192) == "d2x2_w8_r1" and name(96, 11008, 4096) == "d2x2_w8_r1"
+    # ... and 64 x 64 or 64 x 32 blocks, one workgroup per CU, where that makes one round that fills most of the device
+    assert name(128, 8192, 4096) == "d4x4_w8_r1" and name(256, 4096, 4096) == "d4x4_w8_r1" and name(512, 2048, 8192) == "d4x4_w8_r1"
+    assert name(128, 4096, 8192) == "d4x2_w8_r1" and name(192, 4096, 4096) == "d4x4_w8_r1" and name(256, 2048, 4096) == "d4x2_w8_r1"
+    assert name(256, 8192, 4096).startswith("q") and name(512, 4096, 4096).startswith("q") and name(128, 4096, 1024) == "d2x2_w8_r1"
     d22 = qm.config_id("d2x2_w8_r1")
     assert qm.config_supports(d22, 1000, 4096, 4096) and not qm.config_supports(qm.config_id("p2x1_w8_r2k2"), 33, 4096, 4096)
     # a persistent "p" configuration only takes the K its waves hold in registers
@@ -178,22 +182,22 @@ def test_selection_rules():
     assert qm.config_supports(pk, 16, 4096, 4096) and not qm.config_supports(pk, 16, 4096, 4096 + 32) and not qm.config_supports(pk, 17, 4096, 4096)
     assert name(64, 28672, 14336).startswith("q")
     # few tiles, long K: the pipelined kernel with K split over several workgroups per tile
-    code = qm.select_config(128, 8192, 28672)
+    code = qm.select_config(256, 8192, 28672)
     assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
     assert (qm.select_config(8192, 8192, 8192) >> 24) & 0x3F == 1
     # ... which the table's rows were measured with: without a workspace (the plain 7-argument
     # call) such a row's second, unsplit choice runs (measured without one); the cost model
     # for untabled shapes prices the atomics of a split without a workspace and keeps none here
-    for (m, n, k) in [(128, 10240, 8192), (256, 4096, 14336), (512, 8192, 28672), (128, 8192, 28672), (384, 8192, 28672)]:
+    for (m, n, k) in [(256, 8192, 28672), (512, 8192, 28672), (384, 8192, 28672), (640, 4096, 14336), (128, 12288, 28672)]:
         with_ws, without = qm.select_config_ex(m, n, k, workspace=True), qm.select_config_ex(m, n, k, workspace=False)
         assert (with_ws >> 24) & 0x3F > 1 and with_ws == qm.select_config(m, n, k)
-        assert qm.config_name(without & 0xFFFF).startswith(("q", "d2x2")) and (without >> 24) & 0x3F == 1, (m, n, k)
+        assert qm.config_name(without & 0xFFFF).startswith(("q", "d2x2", "d4x4")) and (without >> 24) & 0x3F == 1, (m, n, k)
     assert qm.config_name(qm.select_config_ex(512, 8192, 28672, workspace=False) & 0xFFFF) == "q128x128_w2x2_s9o1"
-    # scaled output, no workspace, long K with a short last K-step: a pipelined configuration
-    # that has the output form, never the generic kernel
-    for (m, n, k) in [(256, 256, 28704), (128, 8192, 28672 + 32), (512, 4096, 14336 + 96)]:
+    # scaled output, no workspace, long K with a short last K-step: a configuration that has
+    # the output form, never the generic kernel
+    for (m, n, k) in [(256, 256, 28704), (128, 8192, 28672 + 32), (512, 4096, 14336 + 96), (640, 4096, 14336 + 32)]:
         code = qm.select_config_ex(m, n, k, workspace=False, scaled=True)
-        assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F == 1, (m, n, k)
+        assert qm.config_name(code & 0xFFFF)[0] in "qd" and (code >> 24) & 0x3F == 1, (m, n, k)
         assert qm.config_has_scaled(code & 0xFFFF)
     assert name(100, 100, 30) == "generic"          # K % 32 != 0: no 16-byte chunks
     assert name(128, 128, 4096, 4) == "generic"     # operands not 16-byte aligned
