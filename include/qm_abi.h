@@ -58,8 +58,8 @@ extern "C" {
  * of benchmarks/mi355x.md's second table) in two cases:
  *   - few output tiles and a long K, which those entry points split over several workgroups
  *     per tile through the workspace: here the best unsplit configuration runs instead.
- *     256 x 8192 x 28672: 70.7 us against 54.9 (1.29x); 512 x 8192 x 28672: 95.9 against
- *     92.5 (1.04x); no other shape of the reference's table splits K;
+ *     Two shapes of the reference's table are left that split K: 256 x 8192 x 28672, 59.3 us
+ *     against 55.8 (1.06x), and 512 x 8192 x 28672, 96-105 us against 92-95 (1.04-1.11x);
  *   - K % 32 != 0, or A or B not 16-byte aligned: no 16-byte loads, the one-thread-per-element
  *     kernel runs (2048 x 4096 x 4100: 3.3 ms, against 44 us on zero-padded copies in a
  *     workspace).  Weight matrices of the reference's table all have K % 32 == 0.

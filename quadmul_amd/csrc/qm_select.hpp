@@ -151,6 +151,25 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         // per workgroup halve that against 16
         return pick(n <= 4096 ? "d2x1_w16_r1" : "d2x2_w8_r1");
     }
+    if (m > 32 && m <= 512 && k >= 2048 && k <= 32768) {
+        // From 33 to a few hundred rows on few columns: blocks of 64 x 64 or 64 x 32 of the same
+        // kernel when that makes one round of workgroups that fills most of the device (eight
+        // waves, one workgroup per CU), or up to two rounds of 64 x 64 blocks on four waves,
+        // two workgroups to a CU -- a workgroup pulls (rows + columns) x K / 2 bytes through its
+        // L1 for rows x columns x K multiply-adds, so the larger block moves half as much per
+        // product.  Measured with B from HBM, M = 64 .. 512, N = 2048 .. 8192, K = 4096 .. 28672,
+        // against the tiles and the 32 x 32 blocks: 128 x 8192 x 8192 15.4 us (64 x 64 tiles:
+        // 19.1), 256 x 4096 x 8192 14.5 (18.8), 512 x 2048 x 4096 8.7 (11.3), 128 x 4096 x 8192
+        // 9.6 on 64 x 32 (32 x 32: 11.1), 64 x 8192 x 4096 6.5 on 64 x 32 (32 x 32: 7.5); in two
+        // rounds 256 x 8192 x 8192 23.1 (128 x 64 tiles: 25.3), 512 x 4096 x 4096 13.5 (15.1).
+        // Beyond two rounds the tiles win, and on a K this long they win with a workspace to
+        // split it through.
+        const long long r64 = (m + 63) / 64, c64 = (n + 63) / 64, c32 = (n + 31) / 32, r32 = (m + 31) / 32;
+        if (r64 * c64 >= 140 && r64 * c64 <= 256) return pick("d4x4_w8_r1");
+        if (r64 * c64 > 256 && r64 * c64 <= 512 && (k <= 16384 || !has_ws)) return pick("d4x4_w4_r1");
+        if (r64 * c32 >= 140 && r64 * c32 <= 256) return pick("d4x2_w8_r1");
+        if (r32 * c64 >= 140 && r32 * c64 <= 256) return pick("d2x4_w8_r1");
+    }
     if (m <= 64) {
         // blocks of 32 rows: 32 x 16 per workgroup while that leaves one workgroup per CU,
         // 32 x 32 (two to a CU) up to about three rounds of them, tiles beyond
@@ -166,22 +185,6 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         // kernel: 114; on zero-padded copies in a workspace: 11.9), 8192 x 8192 x 96 66 us (875; 56).
         const long long wgs = (long long)((m + 31) / 32) * ((n + 31) / 32);
         return pick(wgs > 1024 ? "d2x2_w1_r1" : "d2x2_w8_r1");
-    }
-    if (m <= 512 && k >= 2048 && k <= 32768) {
-        // A few hundred rows on few columns: blocks of 64 x 64 or 64 x 32 of the same kernel, one
-        // workgroup per CU, when that makes one round of workgroups that fills most of the
-        // device -- a workgroup pulls (rows + columns) x K / 2 bytes through its L1 for rows x
-        // columns x K multiply-adds, so the larger block moves half as much per product.
-        // Measured with B from HBM, M = 96 .. 512, N = 2048 .. 8192, K = 4096 .. 28672, against
-        // the tiles and the 32 x 32 blocks: 128 x 8192 x 8192 15.4 us (64 x 64 tiles: 19.1),
-        // 256 x 4096 x 8192 14.5 (18.8), 512 x 2048 x 4096 8.7 (11.3), 128 x 4096 x 8192 9.6 on
-        // 64 x 32 (32 x 32: 11.1).  Two rounds lose to the tiles, except on a long K without a
-        // workspace to split it through.
-        const long long r64 = (m + 63) / 64, c64 = (n + 63) / 64, c32 = (n + 31) / 32, r32 = (m + 31) / 32;
-        if (r64 * c64 >= 140 && r64 * c64 <= 256) return pick("d4x4_w8_r1");
-        if (!has_ws && k >= 8192 && r64 * c64 > 256 && r64 * c64 <= 512) return pick("d4x4_w8_r1");
-        if (r64 * c32 >= 140 && r64 * c32 <= 256) return pick("d4x2_w8_r1");
-        if (r32 * c64 >= 140 && r32 * c64 <= 256) return pick("d2x4_w8_r1");
     }
     if (m <= 256 && k <= 16384) {
         // The same 32 x 32 blocks on a few hundred rows (measured with B from HBM, M = 65 .. 256,
