@@ -151,13 +151,13 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         // per workgroup halve that against 16
         return pick(n <= 4096 ? "d2x1_w16_r1" : "d2x2_w8_r1");
     }
-    if (m > 32 && m <= 512 && k >= 2048 && k <= 32768) {
-        // From 33 to a few hundred rows on few columns: blocks of 64 x 64 or 64 x 32 of the same
+    if (m > 32 && m <= 1024 && k >= 1024 && k <= 32768) {
+        // From 33 to a thousand rows on few columns: blocks of 64 x 64 or 64 x 32 of the same
         // kernel when that makes one round of workgroups that fills most of the device (eight
         // waves, one workgroup per CU), or up to two rounds of 64 x 64 blocks on four waves,
         // two workgroups to a CU -- a workgroup pulls (rows + columns) x K / 2 bytes through its
         // L1 for rows x columns x K multiply-adds, so the larger block moves half as much per
-        // product.  Measured with B from HBM, M = 64 .. 512, N = 2048 .. 8192, K = 4096 .. 28672,
+        // product.  Measured with B from HBM, M = 40 .. 1024, N = 1024 .. 32768, K = 1024 .. 28672,
         // against the tiles and the 32 x 32 blocks: 128 x 8192 x 8192 15.4 us (64 x 64 tiles:
         // 19.1), 256 x 4096 x 8192 14.5 (18.8), 512 x 2048 x 4096 8.7 (11.3), 128 x 4096 x 8192
         // 9.6 on 64 x 32 (32 x 32: 11.1), 64 x 8192 x 4096 6.5 on 64 x 32 (32 x 32: 7.5); in two

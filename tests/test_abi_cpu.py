@@ -167,7 +167,7 @@ def test_selection_rules():
     assert name(3, 28672, 2048) == "p1x1_w8_r2k2" and name(16, 4096, 8192) == "d1x1_w16_r1"
     assert name(32, 11008, 4096) == "p2x1_w8_r2k2" and name(24, 4096, 2048) == "p2x1_w16_r2k1"
     assert name(24, 4096, 8192) == "d2x1_w16_r1" and name(32, 28672, 8192) == "d2x2_w8_r1" and name(20, 2048, 8192) == "d1x1_w16_r1"
-    assert name(40, 4096, 14336) == "d2x2_w8_r1" and name(64, 2048, 4096) == "d2x1_w16_r1" and name(64, 20000, 1024).startswith("q64x")
+    assert name(40, 4096, 14336) == "d2x2_w8_r1" and name(64, 2048, 4096) == "d2x1_w16_r1" and name(64, 40000, 4096).startswith("q")
     # 33 rows and more on enough columns: 64 x 32 and 64 x 64 blocks in one round of workgroups
     assert name(64, 8192, 4096) == "d4x2_w8_r1" and name(64, 11008, 4096) == "d4x4_w8_r1" and name(40, 16384, 8192) == "d4x4_w8_r1"
     # a few hundred rows on few columns: the same 32 x 32 blocks, up to about three rounds of workgroups
@@ -176,7 +176,7 @@ def test_selection_rules():
     assert name(128, 8192, 4096) == "d4x4_w8_r1" and name(256, 4096, 4096) == "d4x4_w8_r1" and name(512, 2048, 8192) == "d4x4_w8_r1"
     assert name(128, 4096, 8192) == "d4x2_w8_r1" and name(192, 4096, 4096) == "d4x4_w8_r1" and name(256, 2048, 4096) == "d4x2_w8_r1"
     # ... or up to two rounds of 64 x 64 blocks on four waves, two workgroups to a CU; tiles beyond
-    assert name(256, 8192, 4096) == "d4x4_w4_r1" and name(512, 4096, 4096) == "d4x4_w4_r1" and name(128, 4096, 1024) == "d2x2_w8_r1"
+    assert name(256, 8192, 4096) == "d4x4_w4_r1" and name(512, 4096, 4096) == "d4x4_w4_r1" and name(128, 4096, 512) == "d2x2_w8_r1"
     assert name(512, 8192, 4096).startswith("q") and name(384, 8192, 28672).startswith("q")
     d22 = qm.config_id("d2x2_w8_r1")
     assert qm.config_supports(d22, 1000, 4096, 4096) and not qm.config_supports(qm.config_id("p2x1_w8_r2k2"), 33, 4096, 4096)
