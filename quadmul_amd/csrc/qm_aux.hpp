@@ -174,6 +174,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitReduceArg
         int32_t *crow = static_cast<int32_t *>(q.C) + (size_t)m * q.N;
         if ((q.N & 3) == 0 && ((uintptr_t)q.C & 15) == 0) {
             *reinterpret_cast<v4i *>(crow + n) = sum;  // n % 4 == 0 and N % 4 == 0: all four inside
+        } else if (n + 3 < q.N) {
+            *reinterpret_cast<v4i_elem_aligned *>(crow + n) = sum;
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
@@ -190,6 +192,8 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitReduceArg
         }
         if ((q.N & 3) == 0 && ((uintptr_t)q.C & 7) == 0) {
             *reinterpret_cast<v2i *>(drow + n) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
+        } else if (n + 3 < q.N) {
+            *reinterpret_cast<v2i_half_aligned *>(drow + n) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
         } else {
 #pragma unroll
             for (int e = 0; e < 4; ++e)

@@ -7,6 +7,12 @@ namespace qm {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
+// The same at the alignment of one element: what a row of C has when N % 4 != 0 (or C itself
+// is not 16-byte aligned).  A store through these is still one global_store_dwordx4 / x2 --
+// the device takes them at any alignment -- where four element-wise stores per lane, 16 bytes
+// apart from the next lane's, ran at a third of the speed (1444 x 31702 x 128: 104 us).
+typedef v4i v4i_elem_aligned __attribute__((aligned(4)));
+typedef v2i v2i_half_aligned __attribute__((aligned(2)));
 
 // Output forms: the exact int32 product, or the product scaled per row and per column in
 // fp32 and rounded to a 16-bit float (the "dequantise on the way out" use the reference's

@@ -231,6 +231,8 @@ gemm_skinny_dma_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int
         if (p.out == OUT_I32) {
             if (vec_ok) {
                 *reinterpret_cast<v4i *>(p.C + at) = s;  // n % 4 == 0 and N % 4 == 0 (with a row stride: N is that stride or differs from it by a multiple of 256): all four inside
+            } else if (n + 3 < p.N) {
+                *reinterpret_cast<v4i_elem_aligned *>(p.C + at) = s;
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
@@ -247,6 +249,8 @@ gemm_skinny_dma_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, const int
             }
             if (vec_ok) {
                 *reinterpret_cast<v2i *>(d) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
+            } else if (n + 3 < p.N) {
+                *reinterpret_cast<v2i_half_aligned *>(d) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
@@ -478,6 +482,8 @@ gemm_skinny_stream_dma_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, co
             if (p.out == OUT_I32) {
                 if (vec_ok) {
                     *reinterpret_cast<v4i *>(p.C + at) = s;
+                } else if (n + 3 < p.N) {
+                    *reinterpret_cast<v4i_elem_aligned *>(p.C + at) = s;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
@@ -494,6 +500,8 @@ gemm_skinny_stream_dma_kernel(const uint8_t *A, const uint8_t *B, int32_t *C, co
                 }
                 if (vec_ok) {
                     *reinterpret_cast<v2i *>(d) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
+                } else if (n + 3 < p.N) {
+                    *reinterpret_cast<v2i_half_aligned *>(d) = v2i{(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)

@@ -626,6 +626,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                 const v2i o = pack16(v);
                 if (vec_ok && n + 3 < p.N) {
                     *reinterpret_cast<v2i *>(drow + n) = o;
+                } else if (n + 3 < p.N) {
+                    *reinterpret_cast<v2i_half_aligned *>(drow + n) = o;
                 } else {
                     if (n < p.N) drow[n] = (uint16_t)o.x;
                     if (n + 1 < p.N) drow[n + 1] = (uint16_t)((uint32_t)o.x >> 16);
@@ -644,6 +646,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     if (n + e < p.N) __hip_atomic_fetch_add(crow + n + e, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             } else if (vec_ok && n + 3 < p.N) {
                 *reinterpret_cast<v4i *>(crow + n) = v;
+            } else if (n + 3 < p.N) {
+                *reinterpret_cast<v4i_elem_aligned *>(crow + n) = v;
             } else {
                 if (n < p.N) crow[n] = v.x;
                 if (n + 1 < p.N) crow[n + 1] = v.y;
