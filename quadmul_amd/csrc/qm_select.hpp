@@ -4,6 +4,7 @@
 // KernelConfig table (kernel.cu:321-385, configs.cu:19-689), which skips unknown shapes.
 // Included by qm_dispatch.hip only, after the launchers of the skinny and dot kernels.
 #pragma once
+#include <cmath>
 #include <cstring>
 
 #include "qm_launch.hpp"
@@ -122,6 +123,104 @@ struct Choice {
     int spread = 0;
 };
 
+// --------------------------------------------------------------------------
+// Fitted cost model (qm_cost_model.inc, written by quadmul_amd/cost_model.py from timings of
+// every candidate on a few hundred random shapes).  A configuration works on items of bm x bn
+// elements of C -- tiles of the pipelined kernel, blocks of the wave-level one -- `slots` of
+// them at a time:
+//     items  = ceil(M / bm) * ceil(N / bn) * ksplit
+//     rounds = blend * ceil(items / slots) + (1 - blend) * max(1, items / slots)
+//     fill   = min(1, items / slots),  ksteps = ceil(ceil(K / 128) / ksplit)
+//     us     = ksteps * (rounds * step_us + fill * busy_us) + rounds * round_us + launch_us
+//              + (N % 4 != 0, ksplit == 1:  rounds * odd_us)
+//              + (pipelined kernel, N % 4 == 0, ksplit == 1:  max(1, items sticking out of C / slots) * ragged_us)
+//              + (wave-level kernel, N * K / 2 > 32 MB, items > slots:  (ceil(M / bm) - 1) * N * K / 2e6 * reread_us)
+//              + (ksplit > 1:  split_us + split_us_per_melem * ksplit * M * N / 1e6)
+// blend = 1: a partly filled last round costs as much as a full one (one workgroup per CU);
+// towards 0: in proportion (several small workgroups per CU: the ones left speed up).
+// busy_us: what a K-step slows down by as the device fills up (shared L2s, fabric, power).
+// odd_us: rows of C that are not 16-byte aligned -- the pipelined kernel then writes every
+// tile after its last K-step.  ragged_us: tiles that stick out of C are written through
+// guarded stores.  reread_us: per megabyte of B that the second and later blocks of rows of
+// the wave-level kernel read again after the L2s (32 MB between them) have lost it.
+// --------------------------------------------------------------------------
+struct CostFit {
+    const char *name;
+    int slots;
+    float blend, step_us, busy_us, round_us, odd_us, ragged_us, reread_us, launch_us;
+};
+static const CostFit g_cost_fits[] = {
+#define QM_COST(name, slots, blend, step, busy, round, odd, ragged, reread, launch) {name, slots, blend, step, busy, round, odd, ragged, reread, launch},
+#define QM_COST_SPLIT(fixed, per_melem)
+#include "qm_cost_model.inc"
+#undef QM_COST
+#undef QM_COST_SPLIT
+};
+static const float g_cost_split[2] = {
+#define QM_COST(name, slots, blend, step, busy, round, odd, ragged, reread, launch)
+#define QM_COST_SPLIT(fixed, per_melem) fixed, per_melem
+#include "qm_cost_model.inc"
+#undef QM_COST
+#undef QM_COST_SPLIT
+};
+
+static double modelled_us(const CostFit &f, const ConfigDesc &d, int m, int n, int k, int ks)
+{
+    const long long rows = (m + d.bm - 1) / d.bm, cols = (n + d.bn - 1) / d.bn;
+    const double items = (double)rows * (double)cols * ks;
+    const double share = items / f.slots;
+    const double rounds = f.blend * std::ceil(share) + (1.0 - f.blend) * (share > 1.0 ? share : 1.0);
+    const double ksteps = (double)(((k + 127) / 128 + ks - 1) / ks);
+    double us = ksteps * (rounds * f.step_us + (share < 1.0 ? share : 1.0) * f.busy_us) + rounds * f.round_us + f.launch_us;
+    if (ks == 1 && (n & 3)) us += rounds * f.odd_us;
+    if (ks == 1 && !(n & 3) && d.kind == KIND_TILE16) {
+        const double sticking_out = (double)(rows * cols - (long long)(m / d.bm) * (n / d.bn));
+        if (sticking_out > 0) us += (sticking_out > f.slots ? sticking_out / f.slots : 1.0) * f.ragged_us;
+    }
+    if (d.kind == KIND_SKINNY && (double)n * k / 2 > 32e6 && items > f.slots) us += (double)(rows - 1) * n * k / 2e6 * f.reread_us;
+    if (ks > 1) us += g_cost_split[0] + g_cost_split[1] * 1e-6 * ks * (double)m * (double)n;
+    return us;
+}
+
+// The cheapest candidate by the model.  `scaled`: the 16-bit float output, which not every
+// pipelined configuration has a kernel for (a K split through the workspace always does: the
+// kernel that adds the partial sums up scales and rounds).
+static Choice modelled_choice(int m, int n, int k, int ptr_align, bool has_ws, bool scaled)
+{
+    Choice best{0, 1, 1};
+    double best_us = 1e300;
+    const int kt = (k + 127) / 128;
+    for (const CostFit &f : g_cost_fits) {
+        const int id = find_config(f.name);
+        if (id < 0 || !config_supports(id, m, n, k, ptr_align)) continue;
+        const ConfigDesc &d = g_configs[id];
+        const bool tile = d.kind == KIND_TILE16;
+        const auto offer = [&](double us, int ks) {
+            if (us < best_us) { best_us = us; best = Choice{id, tile ? 4 : 1, ks}; }
+        };
+        if (!scaled || scaled_launcher(id)) offer(modelled_us(f, d, m, n, k, 1), 1);
+        if (!tile) continue;
+        // Few tiles and a long K: the pipelined kernel can split K over several workgroups per
+        // tile (the splits the autotuner times).
+        const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
+        if (has_ws) {
+            static const int splits[] = {2, 3, 4, 6, 8, 12, 16};
+            for (int ks : splits)
+                if (tiles <= 256 && tiles * ks <= 1024 && kt / ks >= 4) offer(modelled_us(f, d, m, n, k, ks), ks);
+        } else if (!scaled) {
+            // No workspace: the partial sums meet in C through 4-byte atomics, which are slow
+            // enough that splitting only pays when each split keeps a long K of its own
+            // (measured: wins at K = 28672, loses at K = 8192): + a quarter on the K-steps, 3 us
+            // and about 10 ps per element and split (512 x 8192 x 28672 in four splits 253 us,
+            // 170 of them the atomics).
+            int t = 1;
+            while (t < 4 && tiles * t * 2 <= 256 && (k / 128) / (t * 2) >= 48) t *= 2;
+            if (t > 1) offer((double)((kt + t - 1) / t) * (f.step_us + f.busy_us) * 1.25 + f.round_us + f.launch_us + 3.0 + 9.9e-6 * (double)m * (double)n * t, t);
+        }
+    }
+    return best;
+}
+
 static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
 {
     if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
@@ -151,31 +250,23 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         // per workgroup halve that against 16
         return pick(n <= 4096 ? "d2x1_w16_r1" : "d2x2_w8_r1");
     }
-    if (m > 32 && m <= 1024 && k >= 1024 && k <= 32768) {
-        // From 33 to a thousand rows on few columns: blocks of 64 x 64 or 64 x 32 of the same
-        // kernel when that makes one round of workgroups that fills most of the device (eight
-        // waves, one workgroup per CU), or up to two rounds of 64 x 64 blocks on four waves,
-        // two workgroups to a CU -- a workgroup pulls (rows + columns) x K / 2 bytes through its
-        // L1 for rows x columns x K multiply-adds, so the larger block moves half as much per
-        // product.  Measured with B from HBM, M = 40 .. 1024, N = 1024 .. 32768, K = 1024 .. 28672,
-        // against the tiles and the 32 x 32 blocks: 128 x 8192 x 8192 15.4 us (64 x 64 tiles:
-        // 19.1), 256 x 4096 x 8192 14.5 (18.8), 512 x 2048 x 4096 8.7 (11.3), 128 x 4096 x 8192
-        // 9.6 on 64 x 32 (32 x 32: 11.1), 64 x 8192 x 4096 6.5 on 64 x 32 (32 x 32: 7.5); in two
-        // rounds 256 x 8192 x 8192 23.1 (128 x 64 tiles: 25.3), 512 x 4096 x 4096 13.5 (15.1).
-        // Beyond two rounds the tiles win, and on a K this long they win with a workspace to
-        // split it through.
-        const long long r64 = (m + 63) / 64, c64 = (n + 63) / 64, c32 = (n + 31) / 32, r32 = (m + 31) / 32;
-        if (r64 * c64 >= 140 && r64 * c64 <= 256) return pick("d4x4_w8_r1");
-        if (r64 * c64 > 256 && r64 * c64 <= 512 && (k <= 16384 || !has_ws)) return pick("d4x4_w4_r1");
-        if (r64 * c32 >= 140 && r64 * c32 <= 256) return pick("d4x2_w8_r1");
-        if (r32 * c64 >= 140 && r32 * c64 <= 256) return pick("d2x4_w8_r1");
-    }
-    if (m <= 64) {
-        // blocks of 32 rows: 32 x 16 per workgroup while that leaves one workgroup per CU,
-        // 32 x 32 (two to a CU) up to about three rounds of them, tiles beyond
+    if (m <= 64 && k >= 1024) {
+        // 33 to 64 rows (measured with B from HBM, M = 40 and 64, N = 1024 .. 32768, K = 1024 ..
+        // 28672): blocks of 64 x 64 or 64 x 32 of the same kernel when that makes one round of
+        // workgroups that fills most of the device (eight waves, one workgroup per CU) -- a
+        // workgroup pulls (rows + columns) x K / 2 bytes through its L1 for rows x columns x K
+        // multiply-adds, so the larger block moves half as much per product: 64 x 8192 x 4096
+        // 6.5 us on 64 x 32 (32 x 32: 7.5) -- else blocks of 32 rows: 32 x 16 per workgroup while
+        // that leaves one workgroup per CU, 32 x 32 (two to a CU) up to about three rounds.
+        const long long c64 = (n + 63) / 64, c32 = (n + 31) / 32;
+        if (k <= 32768) {
+            if (c64 >= 140 && c64 <= 256) return pick("d4x4_w8_r1");
+            if (c64 > 256 && c64 <= 512 && (k <= 16384 || !has_ws)) return pick("d4x4_w4_r1");
+            if (c32 >= 140 && c32 <= 256) return pick("d4x2_w8_r1");
+            if (2 * c64 >= 140 && 2 * c64 <= 256) return pick("d2x4_w8_r1");   // (two blocks of 32 rows)
+        }
         if (n <= 2048) return pick("d2x1_w16_r1");
         if (n <= 12288) return pick("d2x2_w8_r1");
-        if (n <= 16384 && config_supports(find_config("q64x64_w2x2_s8o2"), m, n, k, ptr_align)) return pick("q64x64_w2x2_s8o2");
     }
     if (k < 128) {
         // A K of one short step (32, 64 or 96) is nothing for the pipelined kernel: it has no
@@ -186,73 +277,11 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         const long long wgs = (long long)((m + 31) / 32) * ((n + 31) / 32);
         return pick(wgs > 1024 ? "d2x2_w1_r1" : "d2x2_w8_r1");
     }
-    if (m <= 256 && k <= 16384) {
-        // The same 32 x 32 blocks on a few hundred rows (measured with B from HBM, M = 65 .. 256,
-        // N = 2048 .. 11008, K = 2048 .. 8192): ahead of the tiles -- no ring to fill, one
-        // workgroup per 32 x 32 block of C over all of K -- up to about three rounds of
-        // workgroups (two to a CU), e.g. 128 x 4096 x 8192 11.4 us against 17.3, 192 x 4096 x 4096
-        // 9.7 against 11.1; level with the 64 x 64 tiles at four rounds, behind them beyond.
-        const long long wgs = (long long)((m + 31) / 32) * ((n + 31) / 32);
-        if (wgs <= 800 || (wgs <= 1040 && m <= 96)) return pick("d2x2_w8_r1");
-    }
 tiles:
-    // Tiles: minimise (rounds of 256 workgroups) x (tile area / relative efficiency),
-    // over the configurations that can run this K.  Efficiencies are measured ratios.
-    // eff: throughput per tile area relative to the 256 x 256 tile with the GPU full (measured)
-    static const struct { const char *name; double eff; } cands[] = {
-        {"q256x256_w2x2_s9o1", 1.00}, {"q256x128_w2x2_s9o1", 0.82}, {"q128x256_w2x2_s9o1", 0.82}, {"q128x128_w2x2_s9o1", 0.60},
-        {"q128x64_w2x2_s6o2", 0.46},  {"q64x128_w2x2_s6o2", 0.44},  {"q64x64_w2x2_s8o2", 0.37},
-    };
-    int best = 0, best_ks = 1;
-    double best_cost = 1e300;
-    for (const auto &c : cands) {
-        const int id = find_config(c.name);
-        if (id < 0 || !config_supports(id, m, n, k, ptr_align)) continue;
-        const ConfigDesc &d = g_configs[id];
-        const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
-        // Few tiles and a long K: the pipelined kernel can split K over several workgroups
-        // per tile.  With a workspace the partial sums cost a second kernel (about 8 us all
-        // told, measured); without one they meet in C through 4-byte atomics, which are slow
-        // enough that splitting only pays when each split keeps a long K of its own
-        // (measured: wins at K = 28672, loses at K = 8192).
-        // Cost in units of 16.5 ps (one K-step of the 256 x 256 tile = 65536): K-steps per
-        // item x tile area / efficiency, plus 4 us per round of workgroups for filling the
-        // ring and writing out, plus the split's own cost.
-        const int kt = (k + 127) / 128;
-        auto cost_of = [&](int ks_) {
-            const double rounds = (double)((tiles * ks_ + 255) / 256);
-            return rounds * ((double)((kt + ks_ - 1) / ks_) * d.bm * d.bn / c.eff + 240000.0) + (ks_ > 1 ? 480000.0 + 0.04 * ks_ * tiles * d.bm * d.bn : 0.0);  // (+ the partial tiles, written and read back at about 6 TB/s)
-        };
-        int ks = 1;
-        double cost = cost_of(1);
-        if (d.kind == KIND_TILE16 && has_ws) {
-            for (int t = 2; t <= 16 && tiles * t <= 256 && kt / t >= 4; ++t)
-                if (cost_of(t) < cost) { cost = cost_of(t); ks = t; }
-        } else if (d.kind == KIND_TILE16) {
-            // (no workspace: the split is kept only where it is priced below the unsplit launch)
-            int t = 1;
-            while (t < 4 && tiles * t * 2 <= 256 && (k / 128) / (t * 2) >= 48) t *= 2;
-            if (t > 1) {
-                // (+ one 4-byte atomic per element and split at about 10 ps each, 0.6 units --
-                // measured: 512 x 8192 x 28672 in four splits 253 us, 170 of them the atomics)
-                const double split_cost = (double)d.bm * d.bn / c.eff * ((kt + t - 1) / t) * 1.25 + 180000.0 + 0.6 * (double)m * (double)n * t;
-                if (split_cost < cost) { cost = split_cost; ks = t; }
-            }
-        }
-        if (cost < best_cost) { best_cost = cost; best = id; best_ks = ks; }
-    }
-    if (m <= 128 && skinny_ok) {
-        // The wave-level split-K kernel has no ring to fill and no second kernel, and wins
-        // while N x K is small.  Measured, in the units above: about 2 us plus, per million
-        // elements of B, 0.24 us with four row blocks (33..64 rows, B from HBM) and 0.38 us
-        // with eight (65..128 rows).
-        const char *name = m > 64 ? "s8x1_w8_u1" : (n >= 8192 ? (k >= 8192 ? "s4x1_w8_u2" : "s4x1_w16_u2") : (k >= 8192 ? "s4x1_w16_u2" : "s4x1_w16_u1"));
-        const int id = find_config(name);
-        const double cost_s = (2.0 + (double)n * (double)k / (m > 64 ? 2.6e6 : 4.2e6)) / 1.65e-5;
-        if (id >= 0 && cost_s < best_cost) return {id, 1, 1};
-    }
-    const int ksplit = best_ks;
-    return {best, 4, ksplit};
+    // Everything else -- from 65 rows, and 33 to 64 rows on a short K or very many columns:
+    // the fitted cost model over the tiles of the pipelined kernel and the blocks of the
+    // wave-level one.
+    return modelled_choice(m, n, k, ptr_align, has_ws, false);
 }
 
 static Choice select_config(int m, int n, int k, int ptr_align, bool has_ws)
@@ -292,19 +321,8 @@ static Choice select_scaled(int m, int n, int k, int ptr_align, bool has_ws)
     // workspace, and the kernel that adds them up scales and rounds
     if (ch.ksplit > 1 && has_ws && g_configs[ch.cfg].kind == KIND_TILE16) return ch;
     if (fast_path_ok(m, n, k, ptr_align)) {
-        int best = -1;
-        double best_cost = 1e300;
-        for (const auto &e : g_scaled_tile16) {
-            const int id = find_config(e.name);
-            if (id < 0 || !config_supports(id, m, n, k, ptr_align)) continue;
-            const ConfigDesc &d = g_configs[id];
-            const long long tiles = (long long)((m + d.bm - 1) / d.bm) * ((n + d.bn - 1) / d.bn);
-            const int area = d.bm * d.bn;
-            const double eff = area >= 256 * 256 ? 1.0 : (area >= 256 * 128 ? 0.82 : (area >= 128 * 128 ? 0.60 : (area >= 128 * 64 ? 0.45 : 0.37)));
-            const double cost = (double)((tiles + 255) / 256) * ((double)((k + 127) / 128) * area / eff + 240000.0);  // as in heuristic()
-            if (cost < best_cost) { best_cost = cost; best = id; }
-        }
-        if (best >= 0) return {best, 4, 1};
+        const Choice c = modelled_choice(m, n, k, ptr_align, has_ws, true);
+        if (c.cfg > 0) return c;
     }
     const Choice h = heuristic(m, n, k, ptr_align, false);
     if (h.ksplit <= 1 && scaled_launcher(h.cfg)) return h;

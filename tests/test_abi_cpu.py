@@ -167,23 +167,27 @@ def test_selection_rules():
     assert name(3, 28672, 2048) == "p1x1_w8_r2k2" and name(16, 4096, 8192) == "d1x1_w16_r1"
     assert name(32, 11008, 4096) == "p2x1_w8_r2k2" and name(24, 4096, 2048) == "p2x1_w16_r2k1"
     assert name(24, 4096, 8192) == "d2x1_w16_r1" and name(32, 28672, 8192) == "d2x2_w8_r1" and name(20, 2048, 8192) == "d1x1_w16_r1"
-    assert name(40, 4096, 14336) == "d2x2_w8_r1" and name(64, 2048, 4096) == "d2x1_w16_r1" and name(64, 40000, 4096).startswith("q")
+    assert name(40, 4096, 14336) == "d2x2_w8_r1" and name(64, 2048, 4096) == "d2x1_w16_r1"
     # 33 rows and more on enough columns: 64 x 32 and 64 x 64 blocks in one round of workgroups
     assert name(64, 8192, 4096) == "d4x2_w8_r1" and name(64, 11008, 4096) == "d4x4_w8_r1" and name(40, 16384, 8192) == "d4x4_w8_r1"
-    # a few hundred rows on few columns: the same 32 x 32 blocks, up to about three rounds of workgroups
-    assert name(128, 2048, 8192) == "d2x2_w8_r1" and name(96, 2048, 4096) == "d2x2_w8_r1" and name(96, 11008, 4096) == "d4x4_w4_r1"
-    # ... and 64 x 64 or 64 x 32 blocks, one workgroup per CU, where that makes one round that fills most of the device
+    # From 65 rows (and 33 to 64 on a short K or very many columns) the fitted cost model
+    # chooses, among the tiles of the pipelined kernel and the blocks of the wave-level one.
+    # A few hundred rows on few columns: 32 x 32 blocks (96 rows are three of them, not two of 64)
+    assert name(128, 2048, 8192) == "d2x2_w8_r1" and name(96, 2048, 4096) == "d2x2_w8_r1" and name(96, 11008, 4096) == "d2x2_w8_r1"
+    assert name(72, 2560, 8192) == "d2x2_w8_r1" and name(96, 5120, 3072) == "d2x4_w8_r1"
+    # ... 64 x 64, 32 x 64 or 64 x 32 blocks, one workgroup per CU, where that makes one round that fills most of the device
     assert name(128, 8192, 4096) == "d4x4_w8_r1" and name(256, 4096, 4096) == "d4x4_w8_r1" and name(512, 2048, 8192) == "d4x4_w8_r1"
-    assert name(128, 4096, 8192) == "d4x2_w8_r1" and name(192, 4096, 4096) == "d4x4_w8_r1" and name(256, 2048, 4096) == "d4x2_w8_r1"
-    # ... or up to two rounds of 64 x 64 blocks on four waves, two workgroups to a CU; tiles beyond
-    assert name(256, 8192, 4096) == "d4x4_w4_r1" and name(512, 4096, 4096) == "d4x4_w4_r1" and name(128, 4096, 512) == "d2x2_w8_r1"
-    assert name(512, 8192, 4096).startswith("q") and name(384, 8192, 28672).startswith("q")
+    assert name(128, 4096, 8192) == "d2x4_w8_r1" and name(192, 4096, 4096) == "d4x4_w8_r1" and name(256, 2048, 4096) == "d2x4_w8_r1"
+    # ... or up to two rounds and a half of 64 x 64 blocks on four waves, two workgroups to a CU; tiles beyond
+    assert name(256, 8192, 4096) == "d4x4_w4_r1" and name(512, 4096, 4096) == "d4x4_w4_r1" and name(64, 40000, 4096) == "d4x4_w4_r1"
+    assert name(128, 4096, 512) == "d4x2_w8_r1" and name(300, 300, 256) == "d1x1_w4_r4"
+    assert name(512, 8192, 4096).startswith("q") and name(384, 8192, 28672).startswith("q") and name(1000, 4096, 4096).startswith("q")
     d22 = qm.config_id("d2x2_w8_r1")
     assert qm.config_supports(d22, 1000, 4096, 4096) and not qm.config_supports(qm.config_id("p2x1_w8_r2k2"), 33, 4096, 4096)
     # a persistent "p" configuration only takes the K its waves hold in registers
     pk = qm.config_id("p1x1_w8_r2k2")
     assert qm.config_supports(pk, 16, 4096, 4096) and not qm.config_supports(pk, 16, 4096, 4096 + 32) and not qm.config_supports(pk, 17, 4096, 4096)
-    assert name(64, 28672, 14336) == "d4x4_w4_r1" and name(64, 40000, 14336).startswith("q")
+    assert name(64, 28672, 14336) == "d4x4_w4_r1" and name(64, 40000, 14336) == "d4x4_w4_r1"
     # few tiles, long K: the pipelined kernel with K split over several workgroups per tile
     code = qm.select_config(256, 8192, 28672)
     assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
@@ -191,7 +195,7 @@ def test_selection_rules():
     # ... which the table's rows were measured with: without a workspace (the plain 7-argument
     # call) such a row's second, unsplit choice runs (measured without one); the cost model
     # for untabled shapes prices the atomics of a split without a workspace and keeps none here
-    for (m, n, k) in [(256, 8192, 28672), (512, 8192, 28672), (384, 8192, 28672), (640, 4096, 14336), (128, 12288, 28672)]:
+    for (m, n, k) in [(256, 8192, 28672), (512, 8192, 28672), (384, 8192, 28672), (640, 4096, 20480), (384, 3072, 20480)]:
         with_ws, without = qm.select_config_ex(m, n, k, workspace=True), qm.select_config_ex(m, n, k, workspace=False)
         assert (with_ws >> 24) & 0x3F > 1 and with_ws == qm.select_config(m, n, k)
         assert qm.config_name(without & 0xFFFF).startswith(("q", "d2x2", "d4x4")) and (without >> 24) & 0x3F == 1, (m, n, k)

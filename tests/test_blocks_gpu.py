@@ -53,7 +53,7 @@ def _check_both_outputs(oracle_mod, a, b, m, n, k, seed, expect_family=None):
 
 
 # (m, the kernel family its blocks of columns run on)
-FAMILIES = [(1, "v"), (2, "v"), (8, "d"), (16, "d"), (20, "p"), (40, "d"), (64, "d"), (100, "d"), (300, "q"), (700, "q")]
+FAMILIES = [(1, "v"), (2, "v"), (8, "d"), (16, "d"), (20, "p"), (40, "d"), (64, "d"), (100, "d"), (300, "d"), (1500, "q")]
 
 
 @pytest.mark.parametrize("m,family", FAMILIES, ids=[f"m{m}" for m, _ in FAMILIES])
@@ -62,7 +62,7 @@ def test_blocks_of_columns_on_every_kernel_family(oracle_mod, operand_limit, m, 
     """B above the limit, A below: blocks of 768 and 256 columns of C (the last one ragged)
     through a row stride of n -- a multiple of four (16-byte stores stay aligned where C is)
     or odd (element by element)."""
-    k = 1024 if m <= 16 else 512
+    k = 1024 if m <= 16 or m >= 1000 else 512
     limit = 800 * (k // 2) if m > 256 else 300 * (k // 2)
     if m * (k // 2) >= limit:   # (A must stay below: raise the limit just above it)
         limit = (m + 1) * (k // 2)
@@ -140,12 +140,13 @@ def test_blocks_of_rows_cut_into_blocks_of_columns(oracle_mod, operand_limit, sh
 def test_blocks_of_rows_keep_their_workspace_use(oracle_mod, operand_limit):
     """A above the limit, B below it: each block of rows is a call of its own and may split K
     through the workspace; the call asks for what its largest block uses."""
-    m, n, k = 700, 256, 8192
-    limit = 300 * (k // 2)
+    m, n, k = 2600, 1024, 28672
+    limit = 1300 * (k // 2)
     operand_limit(limit)
-    assert _blocks(limit, k) == 256
+    assert _blocks(limit, k) == 1280
     need = qm.workspace_bytes(m, n, k)
-    assert need == max(qm.workspace_bytes(256, n, k), qm.workspace_bytes(700 % 256, n, k))
+    assert need == max(qm.workspace_bytes(1280, n, k), qm.workspace_bytes(m % 1280, n, k)) > 0
+    assert (qm.select_config(1280, n, k) >> 24) & 0x3F > 1
     a, b = make_operands(m, n, k, SEED_BASE + 9500)
     _check_both_outputs(oracle_mod, a, b, m, n, k, SEED_BASE + 9501)
 

@@ -365,7 +365,7 @@ def test_auto_choice_splits_k_and_matches(oracle_mod):
     # few tiles, long K: the automatic choice splits K; extension module and wrapper agree with the oracle
     import quadmul
 
-    m, n, k = 128, 2048, 28672
+    m, n, k = 450, 1280, 28672
     code = qm.select_config(m, n, k)
     assert qm.config_name(code & 0xFFFF).startswith("q") and (code >> 24) & 0x3F > 1
     assert qm.workspace_bytes(m, n, k) > 0
@@ -413,7 +413,7 @@ def test_random_shapes_through_the_automatic_choice():
         if i % 10 == 0:
             m, k = int(rng.integers(65, 129)), int(rng.integers(8, 64)) * 128   # the 128-row skinny kernel
         if i % 10 == 5:   # few tiles, long K: the pipelined kernel with K split through a workspace
-            m, n, k = int(rng.integers(129, 600)), int(rng.integers(256, 1024)), int(rng.integers(64, 94)) * 128
+            m, n, k = int(rng.integers(450, 1000)), int(rng.integers(1100, 1500)), int(rng.integers(224, 257)) * 128
         if i % 10 == 7:   # many tiles: the pipelined kernel, persistent grid
             m, n, k = int(rng.integers(700, 1500)), int(rng.integers(3000, 6000)), int(rng.integers(4, 16)) * 128
         a = torch.randint(-8, 8, (m, k), dtype=torch.int8, generator=torch.Generator().manual_seed(1000 + i))

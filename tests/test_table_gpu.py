@@ -125,10 +125,10 @@ def test_first_call_of_a_configuration_inside_graph_capture(with_init):
     set-up (LDS size attribute, residency query, scratch address) must work there -- or have
     been done by qm_init beforehand -- and the replays must be exact.  One shape per kernel family, a K split through the workspace
     included."""
-    shapes = [(1024, 1024, 1024), (512, 768, 2048 + 32), (640, 4096, 14336), (128, 4096, 14336), (16, 4096, 4096), (40, 512, 1024), (1, 512, 4096), (33, 70, 30)]
+    shapes = [(1024, 1024, 1024), (512, 768, 2048 + 32), (640, 4096, 20480), (128, 4096, 14336), (16, 4096, 4096), (40, 512, 1024), (1, 512, 4096), (33, 70, 30)]
     names = {qm.config_name(qm.select_config(m, n, k) & 0xFFFF)[0] for (m, n, k) in shapes}
     assert {"q", "p", "d", "v", "g"} <= names, names
-    assert (qm.select_config(640, 4096, 14336) >> 24) & 0x3F > 1     # the K split through the workspace
+    assert (qm.select_config(640, 4096, 20480) >> 24) & 0x3F > 1     # the K split through the workspace
     code = COLD_CAPTURE.format(root=ROOT, shapes=shapes, with_init=with_init)
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=170)
     assert r.returncode == 0 and "COLD-CAPTURE-OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]

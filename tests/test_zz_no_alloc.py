@@ -39,9 +39,9 @@ def _with_workspace(a_d, b_d, m, n, k):
 # array full of an earlier call's data
 CALLS = [
     ((256, 8192, 28672), "partial tiles of a K split, 32 MiB"),
-    ((640, 4096, 14336), "partial tiles of a K split of three, 30 MiB"),
+    ((640, 4096, 20480), "partial tiles of a K split of three, 30 MiB"),
     ((2048, 4096, 4100), "zero-padded copies of A and B"),
-    ((128, 12288, 28672), "partial tiles of a K split of five"),
+    ((384, 3072, 20480), "partial tiles of a K split of three, 13 MiB"),
     ((200, 300, 1152), "nothing (one launch, no scratch)"),
 ]
 
@@ -79,7 +79,7 @@ def test_static_scratch_matches_caller_workspace_on_calls_in_a_row(oracle_mod):
 def test_static_scratch_twice_on_one_stream_then_smaller(oracle_mod):
     # the same array back to back without a synchronisation in between: stream order is all
     # that separates the second call's writes from the first call's reads
-    (m1, n1, k1), (m2, n2, k2) = (256, 8192, 28672), (640, 4096, 14336)
+    (m1, n1, k1), (m2, n2, k2) = (256, 8192, 28672), (640, 4096, 20480)
     a1, b1 = make_operands(m1, n1, k1, SEED_BASE + 7100)
     a2, b2 = make_operands(m2, n2, k2, SEED_BASE + 7101)
     d1 = (pack_cpu(a1).to(DEV), pack_cpu(b1).to(DEV))
