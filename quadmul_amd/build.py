@@ -15,7 +15,9 @@ CUDAExtension), without torch's source-translation step.
 from __future__ import annotations
 
 import argparse
+import glob
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -70,6 +72,39 @@ def _run(cmd):
     return out
 
 
+# A memory instruction must not read a scalar register within five wait states of a vector
+# instruction that wrote it (v_readlane, v_readfirstlane, a comparison into a register pair).
+# The compiler inserts the wait states for its own memory instructions and cannot for the
+# ones inside asm statements -- the ring's loads and the stores of tiles that stick out of C
+# take a base pointer in scalar registers -- so the generated code is scanned for it.
+_ASM_VMEM = re.compile(r"global_(?:store_dwordx[24]|load_lds_dwordx4)\s.*\bs\[(\d+):(\d+)\]")
+
+
+def scalar_operand_hazards(isa_path: str):
+    """(line number, writer, reader) for every load/store with a scalar base in the device
+    assembly at ``isa_path`` whose base a vector instruction wrote fewer than five wait
+    states before."""
+    lines = open(isa_path).read().split("\n")
+    found = []
+    for i, line in enumerate(lines):
+        m = _ASM_VMEM.search(line)
+        if not m:
+            continue
+        lo, hi = int(m[1]), int(m[2])
+        waited, j = 0, i - 1
+        while j >= 0 and waited < 5:
+            t = lines[j].strip()
+            j -= 1
+            if not t or t[0] in ";." or t.endswith(":"):
+                continue
+            if re.match(r"v_(?:readlane|readfirstlane)_b32 s(?:%d|%d)\b" % (lo, hi), t) or re.match(r"v_cmp\S* s\[%d:%d\]" % (lo, hi), t):
+                found.append((i + 1, t, line.strip()))
+                break
+            nop = re.match(r"s_nop (\d+)", t)
+            waited += int(nop[1]) + 1 if nop else 1
+    return found
+
+
 def build_lib(jobs: int = 8, verbose: bool = False) -> str:
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
@@ -86,16 +121,31 @@ def build_lib(jobs: int = 8, verbose: bool = False) -> str:
              ("qm_scratch.o", ["-c", os.path.join(CSRC, "qm_scratch.hip")])]
     for tu in range(N_TILE_TUS):
         units.append((f"qm_tile_inst_{tu}.o", [f"-DQM_TU={tu}", "-c", os.path.join(CSRC, "qm_tile_inst.hip")]))
-    objs = [os.path.join(OBJDIR, name) for name, _ in units]
+    # (a directory per unit: the compiler's intermediate files, kept for the scan below, are
+    # named after the source file, which the tile units share)
+    objs = [os.path.join(OBJDIR, name[:-2], name) for name, _ in units]
 
     def compile_one(item):
         (name, args), obj = item
-        return _run([HIPCC] + HIP_FLAGS + args + ["-o", obj])
+        shutil.rmtree(os.path.dirname(obj), ignore_errors=True)
+        os.makedirs(os.path.dirname(obj))
+        return _run([HIPCC] + HIP_FLAGS + ["-save-temps=obj"] + args + ["-o", obj])
 
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, 16))) as pool:
         for out in pool.map(compile_one, zip(units, objs)):
             if verbose and out.strip():
                 print(out)
+    hazards = []
+    for obj in objs:
+        for isa in glob.glob(os.path.join(os.path.dirname(obj), "*-amdgcn-amd-amdhsa-gfx950.s")):
+            hazards += [(os.path.basename(os.path.dirname(obj)),) + h for h in scalar_operand_hazards(isa)]
+        for junk in glob.glob(os.path.join(os.path.dirname(obj), "*")):
+            if junk != obj:
+                os.remove(junk)
+    if hazards:
+        raise RuntimeError("quadmul_amd.build: a load or store inside an asm statement reads a scalar register that a vector "
+                           "instruction wrote fewer than five wait states before (unit, line, writer, reader):\n  " +
+                           "\n  ".join(str(h) for h in hazards[:20]) + f"\n  ({len(hazards)} in all)")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs)
     return LIB_PATH
 

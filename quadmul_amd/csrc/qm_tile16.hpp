@@ -209,12 +209,13 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // (readfirstlane: the quotients are computed on the vector ALU; everything derived from
     // them is wave-uniform and belongs in scalar registers)
     //
-    // Items come in two ranges.  [0, nwhole): tiles that lie wholly inside the matrix, when C
-    // takes plain 16-byte stores and K is not split -- their write-out needs no guards and is
-    // folded into the last K-step.  [nwhole, nitems): everything else (the ragged right
-    // column and bottom row of tiles; or all items, when nwhole is 0), written out by the
-    // guarded code after the last K-step.  A workgroup's items ascend, so it runs its whole
-    // tiles first and then the rest: two loops one after the other.
+    // When C takes plain 16-byte stores and K is not split, a tile's write-out is folded into
+    // its last K-step.  The items are then numbered in two ranges: [0, nwhole) the tiles that
+    // lie wholly inside the matrix, [nwhole, nitems) the ragged right column and bottom row of
+    // tiles, whose stores are under the condition that their rows and columns exist.  A
+    // workgroup's items ascend, so it runs its whole tiles first.  Otherwise (nwhole is 0: K
+    // split, odd N, unaligned C) every item is written out by the guarded code after its last
+    // K-step.
     const int ldc = c_stride(p);  // row stride of C in elements (N, unless this call computes a block of columns of a wider C)
     const bool vec_ok = (ldc & 3) == 0 && ((uintptr_t)p.C & (4 * ESZ - 1)) == 0;  // 4 elements per store
     const bool plain_c = vec_ok && ksplit == 1 && ldc < (1 << 21);
@@ -329,6 +330,11 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // M0 first (the slots in between are the wait state the load needs after a write of M0),
     // the load itself follows alone -- five instructions in one slot are more than the shadow
     // of that slot's MFMA hides.  Nothing else in this kernel uses M0.
+    // (These statements read the operand's base pointer from scalar registers.  If the
+    // compiler fetched it into them with a vector instruction just before -- v_readlane, when
+    // it keeps scalar registers in the lanes of a vector one -- the load would have to wait
+    // five wait states, which the compiler sees to for its own memory instructions only: the
+    // build scans the generated code for that and fails if it finds it.)
     auto dma_setup = [&](int piece, int stage_byte) __attribute__((always_inline)) {
         const uint32_t dst = dma_lds + stage_byte +
                              (piece < A_PIECES ? piece * WAVES * 16 * PITCH : Cfg::A_BYTES + (piece - A_PIECES) * WAVES * 16 * PITCH);
@@ -512,11 +518,45 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     const int xp_wr = r * Cfg::XPOSE_PITCH + g * 16, xp_rd = (lane >> 4) * Cfg::XPOSE_PITCH + (lane & 15) * 16;
     const uint32_t xp_wr_lds = lds0 + Cfg::RING_BYTES + wave * Cfg::XPOSE_BYTES + xp_wr;  // the same as an LDS address
     v4i xr[4];
+    // A tile that sticks out of C is written the same way as a whole one, every store with the
+    // lanes switched off whose row or columns do not exist.  The store is issued under a lane
+    // mask set and restored around it, not under a branch: the write-out stays one basic block
+    // (with branches between the MFMA slots the register allocator spills), and the address
+    // stays base register + 32-bit lane offset.  rows_left / cols_left are what the matrix has
+    // from this lane's first row and column of the tile on, in the order the stores below use
+    // (set per item; N % 4 == 0, so a lane's four columns are inside or outside together).
+    // A store whose lanes are all off may or may not count as issued, so the last K-step of
+    // such a tile allows for none of its stores in its wait.  Whole tiles keep their plain
+    // stores (the conditions cost ten instructions a store: 1 to 10 % on whole-tile shapes
+    // when every tile went this way), so the kernel has the K loop three times: whole tiles,
+    // tiles that stick out (`edge`), and the guarded write-out after the last K-step.
+    int rows_left = 0, cols_left = 0;
+    // (The two comparisons sit inside the statement as well: written in C++, the compiler
+    // works all the lane masks of a tile out ahead -- 64 register pairs -- and runs out of scalar
+    // registers.  s_nop 4: the compiler may have produced the base register pair with a vector
+    // instruction just before this statement -- v_readlane, when it keeps scalar registers in
+    // the lanes of a vector one -- and a memory instruction must not read such a register
+    // within five wait states; the compiler sees to that for its own instructions and cannot
+    // for the store in here.)
+    auto store_lanes = [&](char *const base, const uint32_t lane_off, const auto v, auto row_, auto col_) __attribute__((always_inline)) {
+        constexpr int row = decltype(row_)::value, col = decltype(col_)::value;
+        const int rl = rows_left, cl = cols_left;   // (an asm operand cannot name a captured variable)
+        uint64_t saved, on;
+        if constexpr (sizeof(v) == 16)
+            asm volatile("s_nop 4\n\tv_cmp_lt_i32_e32 vcc, %7, %5\n\ts_mov_b64 %1, vcc\n\tv_cmp_lt_i32_e32 vcc, %8, %6\n\ts_and_b64 %1, %1, vcc\n\t"
+                         "s_mov_b64 %0, exec\n\ts_mov_b64 exec, %1\n\tglobal_store_dwordx4 %2, %3, %4\n\ts_mov_b64 exec, %0"
+                         : "=&s"(saved), "=&s"(on) : "v"(lane_off), "v"(v), "s"(base), "v"(rl), "v"(cl), "n"(row), "n"(col) : "memory", "vcc");
+        else
+            asm volatile("s_nop 4\n\tv_cmp_lt_i32_e32 vcc, %7, %5\n\ts_mov_b64 %1, vcc\n\tv_cmp_lt_i32_e32 vcc, %8, %6\n\ts_and_b64 %1, %1, vcc\n\t"
+                         "s_mov_b64 %0, exec\n\ts_mov_b64 exec, %1\n\tglobal_store_dwordx2 %2, %3, %4\n\ts_mov_b64 exec, %0"
+                         : "=&s"(saved), "=&s"(on) : "v"(lane_off), "v"(v), "s"(base), "v"(rl), "v"(cl), "n"(row), "n"(col) : "memory", "vcc");
+    };
     // Whole tile, through the LDS: part t = 0..7 of blocks (ib, 4*grp .. 4*grp+3), one part per
     // MFMA slot.  Parts 0..3 write one block each; the read-back of row quartet k and its
     // store are two parts apart, so the store does not wait for the LDS.
-    auto write_group = [&](auto ib_, auto grp_, auto t_) __attribute__((always_inline)) {
+    auto write_group = [&](auto ib_, auto grp_, auto t_, auto edge_) __attribute__((always_inline)) {
         constexpr int ib = decltype(ib_)::value, grp = decltype(grp_)::value, t = decltype(t_)::value;
+        constexpr bool edge = decltype(edge_)::value;
         auto read_back = [&](auto k_) __attribute__((always_inline)) {
             constexpr int k = decltype(k_)::value;
             xr[k] = *reinterpret_cast<const v4i *>(xp + xp_rd + 4 * k * Cfg::XPOSE_PITCH);
@@ -527,9 +567,11 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             if constexpr (OUT == OUT_I32) {
                 v4i v = xr[k];
                 v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
-                *reinterpret_cast<v4i *>(at + lane_row) = v;
+                if constexpr (edge) store_lanes(at, lane_row, v, std::integral_constant<int, ib * 16 + 4 * k>{}, std::integral_constant<int, grp * 64>{});
+                else *reinterpret_cast<v4i *>(at + lane_row) = v;
             } else {
-                *reinterpret_cast<v2i *>(at + lane_row) = pack16(xr[k]);
+                if constexpr (edge) store_lanes(at, lane_row, pack16(xr[k]), std::integral_constant<int, ib * 16 + 4 * k>{}, std::integral_constant<int, grp * 64>{});
+                else *reinterpret_cast<v2i *>(at + lane_row) = pack16(xr[k]);
             }
         };
         if constexpr (t < 4) {
@@ -557,18 +599,21 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     uint8_t *const xh = smem + Cfg::RING_BYTES + wave * Cfg::XHALF_BYTES;
     const int xh_wr = r * 128 + ((g ^ (r & 7)) << 4);                             // block 2h; block 2h + 1 is 64 bytes (chunk bit 2) away
     const int xh_rd = (lane >> 3) * 128 + (((lane & 7) ^ (lane >> 3)) << 4);      // rows 0..7; rows 8..15: + 1024
-    auto store_half = [&](auto ib_, auto h_, auto k_) __attribute__((always_inline)) {
+    auto store_half = [&](auto ib_, auto h_, auto k_, auto edge_) __attribute__((always_inline)) {
+        constexpr bool edge = decltype(edge_)::value;
         constexpr int ib = decltype(ib_)::value, h = decltype(h_)::value, k = decltype(k_)::value;
         char *const at = tile_c + ((size_t)(ib * 16 + 8 * k) * ldc + h * 32) * ESZ;  // wave-uniform
         if constexpr (OUT == OUT_I32) {
             v4i v = xr[k];
             v.x >>= 8; v.y >>= 8; v.z >>= 8; v.w >>= 8;
-            *reinterpret_cast<v4i *>(at + lane_half) = v;
+            if constexpr (edge) store_lanes(at, lane_half, v, std::integral_constant<int, ib * 16 + 8 * k>{}, std::integral_constant<int, h * 32>{});
+            else *reinterpret_cast<v4i *>(at + lane_half) = v;
         } else {
-            *reinterpret_cast<v2i *>(at + lane_half) = pack16(xr[k]);
+            if constexpr (edge) store_lanes(at, lane_half, pack16(xr[k]), std::integral_constant<int, ib * 16 + 8 * k>{}, std::integral_constant<int, h * 32>{});
+            else *reinterpret_cast<v2i *>(at + lane_half) = pack16(xr[k]);
         }
     };
-    auto write_half = [&](auto ib_, auto h_, auto t_) __attribute__((always_inline)) {
+    auto write_half = [&](auto ib_, auto h_, auto t_, auto edge_) __attribute__((always_inline)) {
         constexpr int ib = decltype(ib_)::value, h = decltype(h_)::value, t = decltype(t_)::value;
         constexpr int pib = h > 0 ? ib : ib - 1, ph = h > 0 ? h - 1 : FN / 2 - 1;  // the half group before this one
         if constexpr (t < 2) {
@@ -580,32 +625,37 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
             } else {
                 *reinterpret_cast<v4i *>(xh + at) = take_block(ib_, std::integral_constant<int, 2 * h + t>{});
             }
-            if constexpr (pib >= 0) store_half(std::integral_constant<int, pib>{}, std::integral_constant<int, ph>{}, t_);
+            if constexpr (pib >= 0) store_half(std::integral_constant<int, pib>{}, std::integral_constant<int, ph>{}, t_, edge_);
         }
         if constexpr (t == 2) xr[0] = *reinterpret_cast<const v4i *>(xh + xh_rd);
         if constexpr (t == 3) xr[1] = *reinterpret_cast<const v4i *>(xh + xh_rd + 1024);
     };
-    auto flush_half = [&]() __attribute__((always_inline)) {
-        store_half(std::integral_constant<int, FM - 1>{}, std::integral_constant<int, FN / 2 - 1>{}, std::integral_constant<int, 0>{});
-        store_half(std::integral_constant<int, FM - 1>{}, std::integral_constant<int, FN / 2 - 1>{}, std::integral_constant<int, 1>{});
+    auto flush_half = [&](auto edge_) __attribute__((always_inline)) {
+        store_half(std::integral_constant<int, FM - 1>{}, std::integral_constant<int, FN / 2 - 1>{}, std::integral_constant<int, 0>{}, edge_);
+        store_half(std::integral_constant<int, FM - 1>{}, std::integral_constant<int, FN / 2 - 1>{}, std::integral_constant<int, 1>{}, edge_);
     };
     // Whole tile, no room in the LDS: block (ib, j) stored as it is, in two parts.
-    auto write_block = [&](auto ib_, auto j_, auto t_) __attribute__((always_inline)) {
+    auto write_block = [&](auto ib_, auto j_, auto t_, auto edge_) __attribute__((always_inline)) {
         constexpr int ib = decltype(ib_)::value, j = decltype(j_)::value, t = decltype(t_)::value;
         if constexpr (t == 0) {
             xr[0] = take_block(ib_, j_);
         } else {
             char *const at = tile_c + ((size_t)(ib * 16) * ldc + j * 16) * ESZ;  // wave-uniform
-            if constexpr (OUT == OUT_I32) *reinterpret_cast<v4i *>(at + lane_blk) = xr[0];
-            else *reinterpret_cast<v2i *>(at + lane_blk) = pack16(xr[0]);
+            if constexpr (decltype(edge_)::value) {
+                if constexpr (OUT == OUT_I32) store_lanes(at, lane_blk, xr[0], std::integral_constant<int, ib * 16>{}, std::integral_constant<int, j * 16>{});
+                else store_lanes(at, lane_blk, pack16(xr[0]), std::integral_constant<int, ib * 16>{}, std::integral_constant<int, j * 16>{});
+            } else {
+                if constexpr (OUT == OUT_I32) *reinterpret_cast<v4i *>(at + lane_blk) = xr[0];
+                else *reinterpret_cast<v2i *>(at + lane_blk) = pack16(xr[0]);
+            }
         }
     };
     // Slot s of 2*FN for the blocks of row ib of a whole tile
-    auto write_whole = [&](auto ib_, auto s_) __attribute__((always_inline)) {
+    auto write_whole = [&](auto ib_, auto s_, auto edge_) __attribute__((always_inline)) {
         constexpr int s = decltype(s_)::value;
-        if constexpr (Cfg::XPOSE) write_group(ib_, std::integral_constant<int, s / 8>{}, std::integral_constant<int, s % 8>{});
-        else if constexpr (Cfg::XHALF) write_half(ib_, std::integral_constant<int, s / 4>{}, std::integral_constant<int, s % 4>{});
-        else write_block(ib_, std::integral_constant<int, s / 2>{}, std::integral_constant<int, s % 2>{});
+        if constexpr (Cfg::XPOSE) write_group(ib_, std::integral_constant<int, s / 8>{}, std::integral_constant<int, s % 8>{}, edge_);
+        else if constexpr (Cfg::XHALF) write_half(ib_, std::integral_constant<int, s / 4>{}, std::integral_constant<int, s % 4>{}, edge_);
+        else write_block(ib_, std::integral_constant<int, s / 2>{}, std::integral_constant<int, s % 2>{}, edge_);
     };
     // Any tile: guarded stores (ragged edges, odd N or unaligned C, K-split partial sums)
     auto write_guarded = [&](auto ib_, auto j_) __attribute__((always_inline)) {
@@ -665,7 +715,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
     // the matrix cores afterwards (row FM-1 is left to the caller).
     auto k_step = [&](const uint32_t bmask, auto bs_tag, auto last_tag) __attribute__((always_inline)) {
         constexpr int bs = decltype(bs_tag)::value;
-        constexpr bool last = decltype(last_tag)::value;
+        constexpr bool last = decltype(last_tag)::value != 0;  // 1: the last step of a whole tile, 2: of one that sticks out of C (`edge`)
+        constexpr bool edge = decltype(last_tag)::value == 2;
         constexpr int SLOTS = 2 * FN;                // MFMAs per sub-step
         constexpr int W = Cfg::W_OPS;
         constexpr int BSHARE = W * FN / FM;          // B widening ops per sub-step
@@ -704,7 +755,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                     });
                 }
                 // -- write-out of the accumulator row finished one sub-step ago --
-                if constexpr (last && i >= 1) write_whole(std::integral_constant<int, i - 1>{}, s_);
+                if constexpr (last && i >= 1) write_whole(std::integral_constant<int, i - 1>{}, s_, std::integral_constant<bool, edge>{});
                 // -- DMA pieces of the step AHEAD of this one, one sub-step apart --
                 // (With a ring of three stages the loads issued in a step must have landed
                 // at its end.  In a last step they all go out in sub-step 0, ahead of the
@@ -768,7 +819,8 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         // (paired ring: an odd step has issued the loads of two steps, all younger than what must
         // have landed; after an even step, which issues none, the youngest load belongs to step
         // s+3 and the one before it to s+2, which must be there)
-        constexpr int pending = (Cfg::PAIR ? (bs == 1 ? 2 * NP : 1) : (AHEAD - 2) * NP) + (last ? (FM - 1) * FN - (Cfg::XHALF ? 2 : 0) : 0);
+        // (a tile that sticks out of C: none of its stores is allowed for, see store_lanes)
+        constexpr int pending = (Cfg::PAIR ? (bs == 1 ? 2 * NP : 1) : (AHEAD - 2) * NP) + (last && !edge ? (FM - 1) * FN - (Cfg::XHALF ? 2 : 0) : 0);
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(pending > 63 ? 63 : pending) : "memory");
         if constexpr (Cfg::PAIR) {
             const int ta = a_ring[0], tb = b_ring[0];
@@ -790,9 +842,20 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
 
     // One item: K-steps in pairs; when the item has an odd number of them, the second of the
     // last pair is the padding step and its B operand is widened to zero.
-    auto run_item = [&](auto whole_) __attribute__((always_inline)) {
-        constexpr bool whole = decltype(whole_)::value;
+    auto run_item = [&](auto mode_) __attribute__((always_inline)) {
+        // mode 1: a whole tile, written out with plain stores inside its last K-step; 2: a tile
+        // that sticks out of C, the same with every store under its lanes' conditions;
+        // 0: guarded stores after the last K-step (K split, or a C that does not take plain
+        // 16-byte stores)
+        constexpr int mode = decltype(mode_)::value;
+        constexpr bool whole = mode != 0, edge = mode == 2;
         locate(c_item, c_m0, c_n0, c_kt0, c_KT);
+        if constexpr (edge) {
+            const int mrem = p.M - c_m0, nrem = p.N - c_n0;
+            if constexpr (Cfg::XPOSE) { rows_left = mrem - wm * Cfg::WM - (lane >> 4); cols_left = nrem - wn * Cfg::WN - (lane & 15) * 4; }
+            else if constexpr (Cfg::XHALF) { rows_left = mrem - wm * Cfg::WM - (lane >> 3); cols_left = nrem - wn * Cfg::WN - (lane & 7) * 4; }
+            else { rows_left = mrem - wm * Cfg::WM - r; cols_left = nrem - wn * Cfg::WN - g * 4; }
+        }
         if constexpr (OUT != OUT_I32) {
             // The item's scales, loaded now and waited for now: the compiler cannot see the
             // asm loads of the ring in the memory counter, so a wait it placed at the first
@@ -843,7 +906,7 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
                            ((size_t)xcd_contiguous_id(c_item, nitems) * WAVES + wave) * (FM * FN * 64) + lane;
         }
         k_step(bmask, std::integral_constant<int, 0>{}, std::false_type{});
-        k_step(full, std::integral_constant<int, 1>{}, std::integral_constant<bool, whole>{});
+        k_step(full, std::integral_constant<int, 1>{}, std::integral_constant<int, mode>{});
         // Let the last MFMAs retire before their accumulators are read (the compiler does not
         // know the asm statements were MFMAs, so the wait is tied to the accumulators written
         // last and cannot be scheduled around); then the rows not written out yet.
@@ -852,10 +915,10 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         });
         if constexpr (whole) {
             static_for<0, 2 * FN>([&](auto s_) {
-                write_whole(std::integral_constant<int, FM - 1>{}, s_);
+                write_whole(std::integral_constant<int, FM - 1>{}, s_, std::integral_constant<bool, edge>{});
                 __builtin_amdgcn_sched_barrier(0);
             });
-            if constexpr (Cfg::XHALF) flush_half();
+            if constexpr (Cfg::XHALF) flush_half(std::integral_constant<bool, edge>{});
         } else {
             static_for<0, FM>([&](auto ib_) {
                 static_for<0, FN>([&](auto j_) {
@@ -872,8 +935,12 @@ gemm_tile16_kernel(const GemmArgs p, const int tiles_m, const int tiles_n, const
         // that asm statements are still writing them.
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     };
-    for (; c_item < nwhole; c_item += G) run_item(std::true_type{});
-    for (; c_item < nitems; c_item += G) run_item(std::false_type{});
+    // (three loops one after the other, each of which may run nothing: with loops in the arms
+    // of a branch instead, the register allocator spills)
+    const int nfolded = __builtin_amdgcn_readfirstlane(plain_c ? nitems : 0);
+    for (; c_item < nwhole; c_item += G) run_item(std::integral_constant<int, 1>{});
+    for (; c_item < nfolded; c_item += G) run_item(std::integral_constant<int, 2>{});
+    for (; c_item < nitems; c_item += G) run_item(std::integral_constant<int, 0>{});
     // drain the DMA before the LDS is released
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }

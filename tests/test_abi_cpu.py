@@ -313,3 +313,33 @@ def test_benchmark_table_rows_name_the_kernels_the_library_chooses():
         seen.add((m, n, k))
         assert kernel == chosen, f"benchmarks/mi355x.md row {m}x{n}x{k} names {kernel}, the library chooses {chosen}: regenerate the table"
     assert seen == set(REFERENCE_SHAPES), "the table must cover the reference's 42 shapes (kernel.cu:343-384)"
+
+
+def test_the_build_scans_for_scalar_operands_written_just_before_an_asm_load_or_store(tmp_path):
+    """A memory instruction inside an asm statement that reads a scalar register fewer than
+    five wait states after a vector instruction wrote it: quadmul_amd.build's scan finds it
+    (the compiler keeps that distance for its own memory instructions only)."""
+    from quadmul_amd.build import scalar_operand_hazards
+
+    isa = tmp_path / "unit.s"
+    isa.write_text("\n".join([
+        "\tv_readlane_b32 s10, v193, 49",
+        "\tv_readlane_b32 s11, v193, 50",
+        "\t;;#ASMSTART",
+        "\tglobal_load_lds_dwordx4 v156, s[10:11]",            # one wait state after the write: found
+        "\t;;#ASMEND",
+        "\tv_readlane_b32 s5, v1, 3",
+        "\ts_nop 4",
+        "\tglobal_store_dwordx4 v118, v[72:75], s[4:5]",      # five wait states: fine
+        "\tv_readfirstlane_b32 s20, v7",
+        "\tv_add_u32_e32 v1, v2, v3",
+        "\ts_mov_b64 s[30:31], exec",
+        "\tglobal_store_dwordx2 v118, v[72:73], s[20:21]",    # three: found
+        "\ts_add_u32 s40, s2, s3",
+        "\tglobal_store_dwordx4 v118, v[72:75], s[40:41]",    # written by a scalar instruction: fine
+        "\tv_cmp_ne_u32_e64 s[50:51], 0, v0",
+        "\tglobal_store_dwordx4 v1, v[2:5], off",             # no scalar operand
+        ""]))
+    found = scalar_operand_hazards(str(isa))
+    assert [f[0] for f in found] == [4, 12], found
+    assert "v_readlane_b32 s11" in found[0][1] and "v_readfirstlane_b32 s20" in found[1][1]
