@@ -67,7 +67,6 @@ CANDIDATES = [
 ]
 SLOTS = (256, 512, 1024)
 BLENDS = (0.0, 0.25, 0.5, 0.75, 1.0)
-KSPLITS = (2, 3, 4, 6, 8, 12, 16)   # what the tuner times (autotune.tune_shape) and heuristic() considers
 
 LARGE = dict(m=[72, 96, 128, 160, 200, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1280, 1536, 2048, 2560, 3072, 4096, 6144, 8192],
              n=[1024, 1536, 2048, 2560, 3072, 4096, 5120, 6144, 8192, 11008, 14336, 20480, 28672],

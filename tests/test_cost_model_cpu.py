@@ -3,6 +3,7 @@ the committed numbers are the fit of the committed timings, the built library ev
 same formula, and its choices stay close to the best measured candidate on every shape of
 those timings.  The reference has no counterpart: it skips shapes outside its table
 (kernel.cu:340-385).  No GPU: the timings are data, the choice is host code."""
+import math
 import os
 import re
 
@@ -67,10 +68,10 @@ def test_the_choices_stay_close_to_the_best_measured_candidate():
     rows = cm.load(DATA)
     reg = cm.regret(rows, cm.library_choice)
     assert len(reg) >= 0.95 * len(rows)          # (the choice was among the timed variants)
-    geomean = cm.math.exp(sum(cm.math.log(x[0]) for x in reg) / len(reg))
+    geomean = math.exp(sum(math.log(x[0]) for x in reg) / len(reg))
     assert geomean < 1.02, cm.summarise("library", reg)
     assert reg[0][0] < 1.4, reg[0]
     assert sum(x[0] > 1.05 for x in reg) <= 0.13 * len(reg), cm.summarise("library", reg)
     # shapes whose sizes are multiples of what the kernels work in (the first three collections)
     grid = [x for x in reg if x[1] % 8 == 0 and x[2] % 128 == 0 and x[3] % 128 == 0]
-    assert len(grid) >= 180 and cm.math.exp(sum(cm.math.log(x[0]) for x in grid) / len(grid)) < 1.012
+    assert len(grid) >= 180 and math.exp(sum(math.log(x[0]) for x in grid) / len(grid)) < 1.012
