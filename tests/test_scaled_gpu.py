@@ -246,3 +246,46 @@ def test_scaled_k_padded_through_the_workspace():
             qm.gemm_scaled(a_d, b_d, d, m, n, k, rs_d, cs_d, workspace=ws)
             torch.cuda.synchronize()
             assert torch.equal(d.view(torch.int16), want.view(torch.int16)), (dtype, ws)
+
+
+@pytest.mark.parametrize("shape", [(700, 1300, 512), (1290, 520, 384), (2100, 2052, 256 + 32), (300, 4100, 1024)], ids=lambda s: "x".join(map(str, s)))
+def test_tiles_that_stick_out_of_c_on_every_pipelined_configuration(oracle_mod, shape):
+    """N % 4 == 0 and an aligned C: whole tiles and tiles that stick out of the matrix (a
+    ragged bottom row, a ragged right column, the corner) in one launch, several items per
+    workgroup -- the write-out inside the last K-step with its stores under lane masks --
+    for the int32 output and both 16-bit ones, with and without the one-item-per-workgroup
+    launch, against the oracle; and the memory around C and D stays as it was."""
+    m, n, k = shape
+    a, b = make_operands(m, n, k, SEED_BASE + 7600 + m)
+    ap, bp = pack_cpu(a), pack_cpu(b)
+    rs, cs = make_scales(m, n, SEED_BASE + 7700 + m)
+    c = oracle_mod.gemm_i4(ap.numpy(), bp.numpy())
+    a_d, b_d, rs_d, cs_d = ap.to(DEV), bp.to(DEV), rs.to(DEV), cs.to(DEV)
+    want16 = {out: oracle_mod.scale_round16(c, rs.numpy(), cs.numpy(), out) for _, out in DTYPES}
+    pad = 4096    # elements either side of the output that must not change
+    ran = 0
+    for cfg, name in enumerate(qm.config_names()):
+        if not name.startswith("q") or not qm.config_supports(cfg, m, n, k):
+            continue
+        bm, bn = (int(x) for x in name[1:].split("_")[0].split("x"))
+        assert m % bm or n % bn, (name, shape)          # (some tile sticks out)
+        for gm, spread in [(1, 0), (4, 0), (2, 1)]:
+            code = cfg | (gm << 16) | (spread << 30)
+            buf = torch.full((m * n + 2 * pad,), 0x7F7F7F7F, dtype=torch.int32, device=DEV)
+            c_d = buf[pad:pad + m * n].view(m, n)
+            qm.gemm_cfg(a_d, b_d, c_d, m, n, k, code)
+            torch.cuda.synchronize()
+            bad = oracle_mod.compare(c_d.cpu().numpy(), c)
+            assert bad == -1, f"{name} group_m={gm} spread={spread}: first mismatch at flat index {bad} (row {bad // n}, column {bad % n})"
+            assert (buf[:pad] == 0x7F7F7F7F).all() and (buf[pad + m * n:] == 0x7F7F7F7F).all(), name
+            if not qm.config_has_scaled(cfg):
+                continue
+            for dtype, out in DTYPES:
+                buf16 = torch.full((m * n + 2 * pad,), float("nan"), dtype=dtype, device=DEV)
+                d_d = buf16[pad:pad + m * n].view(m, n)
+                qm.gemm_scaled(a_d, b_d, d_d, m, n, k, rs_d, cs_d, code)
+                torch.cuda.synchronize()
+                assert (bits(d_d) == want16[out]).all(), f"{name} {dtype} group_m={gm} spread={spread}"
+                assert torch.isnan(buf16[:pad]).all() and torch.isnan(buf16[pad + m * n:]).all(), name
+        ran += 1
+    assert ran >= 8
