@@ -225,13 +225,19 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
 {
     if (!fast_path_ok(m, n, k, ptr_align)) return {0, 1, 1};
     // Up to 64 rows: chosen on measurements with B streamed from HBM (launches rotating over
-    // copies of B), M = 1 .. 64, N = 2048 .. 28672, K = 2048 .. 14336.
+    // copies of B), M = 1 .. 64, N = 2048 .. 57344, K = 2048 .. 28672.
     const auto pick = [](const char *name) { const int id = find_config(name); return Choice{id >= 0 ? id : 0, 1, 1}; };
     const bool skinny_ok = m < (1 << 24) && n < (1 << 24);  // (their 24-bit row arithmetic, see config_supports)
     if (!skinny_ok) goto tiles;
     if (m <= 2) {
-        // no matrix core: v_dot8_i32_i4 on the packed bytes as they are
-        if (m == 1) return pick(k <= 2048 ? "v1x1_w8_u4" : (k <= 4096 ? "v1x1_w4_u8" : "v1x1_w16_u2"));
+        // The persistent kernel of the rows above, sixteen waves holding a K of 8192 between
+        // them, is ahead of the dot kernel on that K and many columns even with one row
+        // (1 x 8192 x 8192 7.0 us against 7.8, 1 x 10240 x 8192 8.3 against 9.2, 1 x 57344 x 8192 36.2
+        // against 37.5).
+        if (k > 4096 && k <= 8192 && n >= 8192) return pick("p1x1_w16_r2k2");
+        // no matrix core: v_dot8_i32_i4 on the packed bytes as they are (four waves of eight
+        // chunk pairs again on a very long K: 1 x 8192 x 28672 17.9 us against 19.1)
+        if (m == 1) return pick(k <= 2048 ? "v1x1_w8_u4" : (k <= 4096 || k > 16384 ? "v1x1_w4_u8" : "v1x1_w16_u2"));
         return pick(k <= 4096 ? "v2x1_w8_u4" : "v2x1_w16_u2");
     }
     if (m <= 16) {
@@ -239,9 +245,15 @@ static Choice heuristic(int m, int n, int k, int ptr_align, bool has_ws)
         // while the waves hold all of K
         if (k <= 4096) return pick(k > 2048 || n >= 8192 ? "p1x1_w8_r2k2" : "d1x1_w16_r1");
         if (k <= 8192 && n >= 8192) return pick("p1x1_w16_r2k2");
+        // a very long K: every workgroup re-reads A over all of it; 32 columns per workgroup
+        // halve that (16 x 8192 x 28672 19.1 us against 21.7)
+        if (k > 16384) return pick("d1x2_w8_r2");
         return pick("d1x1_w16_r1");
     }
     if (m <= 32) {
+        // tens of thousands of columns on a long K: one wave per workgroup, thousands of them
+        // (32 x 57344 x 8192 39.9 us against 49.2 on eight waves)
+        if (k > 4096 && n >= 32768) return pick("d2x2_w1_r1");
         if (k <= 2048) return pick("p2x1_w16_r2k1");
         // few column blocks and a long K: two blocks of 16 rows each double the workgroups
         if (n <= 2048) return pick("d1x1_w16_r1");

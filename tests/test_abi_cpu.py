@@ -163,6 +163,11 @@ def test_selection_rules():
     assert name(16, 4096, 4096) == "p1x1_w8_r2k2" and name(64, 4096, 4096) == "d2x2_w8_r1"
     assert name(1, 4096, 4096) == "v1x1_w4_u8" and name(1, 11008, 2048) == "v1x1_w8_u4" and name(2, 5120, 5120) == "v2x1_w16_u2"   # dot-product kernel
     assert name(1, 4096, 8192) == "v1x1_w16_u2" and name(2, 4096, 4096) == "v2x1_w8_u4"
+    # one or two rows on a K of 8192 and many columns: the persistent MFMA kernel is ahead of the dot kernel;
+    # four waves of eight chunk pairs again on a very long K
+    assert name(1, 8192, 8192) == "p1x1_w16_r2k2" and name(2, 57344, 8192) == "p1x1_w16_r2k2" and name(1, 8192, 28672) == "v1x1_w4_u8"
+    # a very long K on up to 16 rows: 32 columns per workgroup; tens of thousands of columns on up to 32 rows: one wave per workgroup
+    assert name(16, 8192, 28672) == "d1x2_w8_r2" and name(32, 57344, 8192) == "d2x2_w1_r1"
     assert name(9, 28672, 14336) == "d1x1_w16_r1" and name(9, 11008, 8192) == "p1x1_w16_r2k2" and name(12, 2048, 2048) == "d1x1_w16_r1"
     assert name(3, 28672, 2048) == "p1x1_w8_r2k2" and name(16, 4096, 8192) == "d1x1_w16_r1"
     assert name(32, 11008, 4096) == "p2x1_w8_r2k2" and name(24, 4096, 2048) == "p2x1_w16_r2k1"
