@@ -14,6 +14,7 @@ kernel, of bm x bn elements of C):
     fill   = min(1, items / slots)
     ksteps = ceil(ceil(K / 128) / ksplit)
     us     = ksteps * (rounds * step_us + fill * busy_us) + rounds * round_us + launch_us
+             [+ ksteps * rounds * skew_us                       when K % 256 != 0]
              [+ rounds * odd_us                                 when N % 4 != 0 and ksplit == 1]
              [+ max(1, ragged items / slots) * ragged_us        pipelined kernel, N % 4 == 0, ksplit == 1]
              [+ (ceil(M / bm) - 1) * N * K / 2e6 * reread_us    wave-level kernel, N * K / 2 > 32 MB, items > slots]
@@ -28,8 +29,11 @@ power); ``odd_us`` is added per round when N % 4 != 0 (rows of C that are not 16
 the pipelined kernel then writes every tile after its last K-step, none of it folded into
 that step); ``ragged_us`` per round of tiles that stick out of C (they are written through
 guarded stores after the last K-step); ``reread_us`` per megabyte of B that the second and
-later blocks of rows of the wave-level kernel read again after the L2s have lost it.
-The nine numbers per configuration and the two of the K split are least-squares fits
+later blocks of rows of the wave-level kernel read again after the L2s have lost it;
+``skew_us`` is what a K-step costs more when the rows of A and B are not whole 128-byte
+lines (K % 256 != 0: every 128-byte run of a row then lies across two cache lines -- 20 to 25 %
+per step on the wave-level kernel, 6 to 15 % on the pipelined one).
+The ten numbers per configuration and the two of the K split are least-squares fits
 (relative error) to timings of every candidate on a few hundred random shapes:
 
     python -m quadmul_amd.cost_model collect --seed 11 --count 60 --domain large --data benchmarks/cost_model_data.jsonl
@@ -102,7 +106,8 @@ def features(name: str, m: int, n: int, k: int, ksplit: int, slots: int, blend: 
             ragged = max(1.0, sticking_out / slots)
     if name[0] == "d" and n * k / 2 > REREAD_BYTES and items > slots:
         reread = (rows - 1) * n * k / 2e6
-    return [rounds * ksteps, rounds, 1.0, min(1.0, items / slots) * ksteps, odd, ragged, reread]
+    skew = rounds * ksteps if k % 256 else 0.0
+    return [rounds * ksteps, rounds, 1.0, min(1.0, items / slots) * ksteps, odd, ragged, reread, skew]
 
 
 def load(paths: str) -> List[Dict]:
@@ -146,7 +151,7 @@ def fit(rows: List[Dict], candidates: Iterable[str] = CANDIDATES) -> Dict:
                     best = (err, slots, blend, coef)
         par[name] = {"slots": best[1], "blend": best[2], "step_us": float(best[3][0]), "round_us": float(best[3][1]),
                      "launch_us": float(best[3][2]), "busy_us": float(best[3][3]), "odd_us": float(best[3][4]), "ragged_us": float(best[3][5]),
-                     "reread_us": float(best[3][6]), "rms": best[0], "points": len(pts)}
+                     "reread_us": float(best[3][6]), "skew_us": float(best[3][7]), "rms": best[0], "points": len(pts)}
     xs, ys = [], []
     for r in rows:
         for (name, ks), us in times_of(r).items():
@@ -161,7 +166,7 @@ def predict(par: Dict, model: Optional[Dict], name: str, m: int, n: int, k: int,
     p = par[name]
     ks = ksplit_items or ksplit
     f = features(name, m, n, k, ks, p["slots"], p["blend"])
-    us = f[0] * p["step_us"] + f[1] * p["round_us"] + p["launch_us"] + f[3] * p["busy_us"] + f[4] * p["odd_us"] + f[5] * p["ragged_us"] + f[6] * p["reread_us"]
+    us = f[0] * p["step_us"] + f[1] * p["round_us"] + p["launch_us"] + f[3] * p["busy_us"] + f[4] * p["odd_us"] + f[5] * p["ragged_us"] + f[6] * p["reread_us"] + f[7] * p["skew_us"]
     if model is not None and ksplit > 1:
         us += model["split_us"] + model["split_us_per_melem"] * ksplit * m * n / 1e6
     return us
@@ -204,7 +209,7 @@ def emit(model: Dict, path: str, rows: List[Dict]) -> None:
         "// Fitted cost model of the kernel choice for shapes outside the per-shape table:",
         "// QM_COST(\"config name\", slots, blend, us per K-step of 128 and round, us per K-step with the device full,",
         "//         us per round, us more per round when N % 4 != 0, us per round of tiles that stick out of C,",
-        "//         us per MB of B read again, us per launch)",
+        "//         us per MB of B read again, us more per K-step and round when K % 256 != 0, us per launch)",
         "// and QM_COST_SPLIT(us per K split, us per million partial elements).  The formula is in",
         "// heuristic() (qm_select.hpp) and in quadmul_amd/cost_model.py, which wrote this file from",
         f"// timings of every candidate on {len(rows)} shapes on MI355X.",
@@ -213,7 +218,7 @@ def emit(model: Dict, path: str, rows: List[Dict]) -> None:
     for name in CANDIDATES:
         p = model["configs"].get(name)
         if p:
-            lines.append(f"QM_COST(\"{name}\", {p['slots']}, {p['blend']:.2f}f, {p['step_us']:.4f}f, {p['busy_us']:.4f}f, {p['round_us']:.3f}f, {p['odd_us']:.3f}f, {p['ragged_us']:.3f}f, {p['reread_us']:.4f}f, {p['launch_us']:.3f}f)"
+            lines.append(f"QM_COST(\"{name}\", {p['slots']}, {p['blend']:.2f}f, {p['step_us']:.4f}f, {p['busy_us']:.4f}f, {p['round_us']:.3f}f, {p['odd_us']:.3f}f, {p['ragged_us']:.3f}f, {p['reread_us']:.4f}f, {p['skew_us']:.4f}f, {p['launch_us']:.3f}f)"
                          f"  // rms {100*p['rms']:.1f} % over {p['points']} shapes")
     lines.append(f"QM_COST_SPLIT({model['split_us']:.3f}f, {model['split_us_per_melem']:.4f}f)")
     with open(path, "w") as f:
@@ -286,7 +291,7 @@ def main(argv=None) -> int:
     if a.what == "fit":
         model = fit(rows)
         for name, p in model["configs"].items():
-            print(f"{name:22s} slots {p['slots']:4d} blend {p['blend']:.2f} step {p['step_us']:.4f} busy {p['busy_us']:.4f} round {p['round_us']:.2f} odd {p['odd_us']:.2f} ragged {p['ragged_us']:.2f} reread {p['reread_us']:.4f} launch {p['launch_us']:.2f}"
+            print(f"{name:22s} slots {p['slots']:4d} blend {p['blend']:.2f} step {p['step_us']:.4f} busy {p['busy_us']:.4f} round {p['round_us']:.2f} odd {p['odd_us']:.2f} ragged {p['ragged_us']:.2f} reread {p['reread_us']:.4f} skew {p['skew_us']:.4f} launch {p['launch_us']:.2f}"
                   f"  rms {100*p['rms']:.1f} %")
         print(f"K split: {model['split_us']:.2f} us + {model['split_us_per_melem']:.3f} us per million partial elements")
         reg = regret(rows, lambda r: choose(model, r))

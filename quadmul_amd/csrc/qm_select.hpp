@@ -132,6 +132,7 @@ struct Choice {
 //     rounds = blend * ceil(items / slots) + (1 - blend) * max(1, items / slots)
 //     fill   = min(1, items / slots),  ksteps = ceil(ceil(K / 128) / ksplit)
 //     us     = ksteps * (rounds * step_us + fill * busy_us) + rounds * round_us + launch_us
+//              + (K % 256 != 0:  ksteps * rounds * skew_us)
 //              + (N % 4 != 0, ksplit == 1:  rounds * odd_us)
 //              + (pipelined kernel, N % 4 == 0, ksplit == 1:  max(1, items sticking out of C / slots) * ragged_us)
 //              + (wave-level kernel, N * K / 2 > 32 MB, items > slots:  (ceil(M / bm) - 1) * N * K / 2e6 * reread_us)
@@ -143,21 +144,23 @@ struct Choice {
 // tile after its last K-step.  ragged_us: tiles that stick out of C are written through
 // guarded stores.  reread_us: per megabyte of B that the second and later blocks of rows of
 // the wave-level kernel read again after the L2s (32 MB between them) have lost it.
+// skew_us: rows of A and B that are not whole 128-byte lines -- every 128-byte run of a row
+// then lies across two cache lines.
 // --------------------------------------------------------------------------
 struct CostFit {
     const char *name;
     int slots;
-    float blend, step_us, busy_us, round_us, odd_us, ragged_us, reread_us, launch_us;
+    float blend, step_us, busy_us, round_us, odd_us, ragged_us, reread_us, skew_us, launch_us;
 };
 static const CostFit g_cost_fits[] = {
-#define QM_COST(name, slots, blend, step, busy, round, odd, ragged, reread, launch) {name, slots, blend, step, busy, round, odd, ragged, reread, launch},
+#define QM_COST(name, slots, blend, step, busy, round, odd, ragged, reread, skew, launch) {name, slots, blend, step, busy, round, odd, ragged, reread, skew, launch},
 #define QM_COST_SPLIT(fixed, per_melem)
 #include "qm_cost_model.inc"
 #undef QM_COST
 #undef QM_COST_SPLIT
 };
 static const float g_cost_split[2] = {
-#define QM_COST(name, slots, blend, step, busy, round, odd, ragged, reread, launch)
+#define QM_COST(name, slots, blend, step, busy, round, odd, ragged, reread, skew, launch)
 #define QM_COST_SPLIT(fixed, per_melem) fixed, per_melem
 #include "qm_cost_model.inc"
 #undef QM_COST
@@ -172,6 +175,7 @@ static double modelled_us(const CostFit &f, const ConfigDesc &d, int m, int n, i
     const double rounds = f.blend * std::ceil(share) + (1.0 - f.blend) * (share > 1.0 ? share : 1.0);
     const double ksteps = (double)(((k + 127) / 128 + ks - 1) / ks);
     double us = ksteps * (rounds * f.step_us + (share < 1.0 ? share : 1.0) * f.busy_us) + rounds * f.round_us + f.launch_us;
+    if (k & 255) us += ksteps * rounds * f.skew_us;
     if (ks == 1 && (n & 3)) us += rounds * f.odd_us;
     if (ks == 1 && !(n & 3) && d.kind == KIND_TILE16) {
         const double sticking_out = (double)(rows * cols - (long long)(m / d.bm) * (n / d.bn));

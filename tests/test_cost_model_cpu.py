@@ -18,7 +18,7 @@ INC = os.path.join(ROOT, "quadmul_amd", "csrc", "qm_cost_model.inc")
 def _committed():
     text = open(INC).read()
     rows = {}
-    for mm in re.finditer(r'^QM_COST\("([^"]+)", (\d+)((?:, [-\d.]+f){8})\)', text, re.M):
+    for mm in re.finditer(r'^QM_COST\("([^"]+)", (\d+)((?:, [-\d.]+f){9})\)', text, re.M):
         rows[mm[1]] = (int(mm[2]),) + tuple(float(x.rstrip("f")) for x in mm[3].split(", ")[1:])
     sp = re.search(r"^QM_COST_SPLIT\(([-\d.]+)f, ([-\d.]+)f\)", text, re.M)
     return rows, (float(sp[1]), float(sp[2]))
@@ -36,7 +36,7 @@ def test_the_committed_numbers_are_the_fit_of_the_committed_timings():
     inc, split = _committed()
     assert set(inc) == set(model["configs"]) == set(cm.CANDIDATES)
     for name, p in model["configs"].items():
-        want = (p["slots"], p["blend"], p["step_us"], p["busy_us"], p["round_us"], p["odd_us"], p["ragged_us"], p["reread_us"], p["launch_us"])
+        want = (p["slots"], p["blend"], p["step_us"], p["busy_us"], p["round_us"], p["odd_us"], p["ragged_us"], p["reread_us"], p["skew_us"], p["launch_us"])
         assert inc[name][0] == want[0] and all(abs(a - b) < 6e-4 for a, b in zip(inc[name][1:], want[1:])), (name, inc[name], want)
     assert abs(split[0] - model["split_us"]) < 6e-4 and abs(split[1] - model["split_us_per_melem"]) < 6e-5
     # every candidate is a configuration the library has
