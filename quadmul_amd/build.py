@@ -31,7 +31,7 @@ LIBDIR = os.path.join(PKG, "lib")
 OBJDIR = os.path.join(PKG, "build")
 LIB_PATH = os.path.join(LIBDIR, "libqm_hip.so")
 PROBE_PATH = os.path.join(LIBDIR, "libqm_probe.so")
-N_TILE_TUS = 12
+N_TILE_TUS = 14
 
 HIPCC = os.environ.get("HIPCC", shutil.which("hipcc") or "/opt/rocm/bin/hipcc")
 HIP_FLAGS = [
@@ -119,8 +119,9 @@ def build_lib(jobs: int = 8, verbose: bool = False) -> str:
         print(f"quadmul_amd.build: WARNING: {msg}; run `pytest tests -m gpu` before trusting results", file=sys.stderr)
     units = [("qm_dispatch.o", [f'-DQM_COMPILER_VERSION="{ver}"', "-mllvm", "-amdgpu-kernarg-preload-count=16", "-c", os.path.join(CSRC, "qm_dispatch.hip")]),
              ("qm_scratch.o", ["-c", os.path.join(CSRC, "qm_scratch.hip")])]
-    for tu in range(N_TILE_TUS):
-        units.append((f"qm_tile_inst_{tu}.o", [f"-DQM_TU={tu}", "-c", os.path.join(CSRC, "qm_tile_inst.hip")]))
+    # (the units with the scaled-output kernels, 6 and up, take longest: they go first)
+    units = [(f"qm_tile_inst_{tu}.o", [f"-DQM_TU={tu}", "-c", os.path.join(CSRC, "qm_tile_inst.hip")])
+             for tu in sorted(range(N_TILE_TUS), key=lambda t: (t < 6, t))] + units
     # (a directory per unit: the compiler's intermediate files, kept for the scan below, are
     # named after the source file, which the tile units share)
     objs = [os.path.join(OBJDIR, name[:-2], name) for name, _ in units]

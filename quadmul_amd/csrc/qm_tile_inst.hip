@@ -95,6 +95,8 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16_9(...)
 #define QM_PICK16_10(...)
 #define QM_PICK16_11(...)
+#define QM_PICK16_12(...)
+#define QM_PICK16_13(...)
 #define QM_PICK16S_0(...)
 #define QM_PICK16S_1(...)
 #define QM_PICK16S_2(...)
@@ -107,6 +109,8 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16S_9(...)
 #define QM_PICK16S_10(...)
 #define QM_PICK16S_11(...)
+#define QM_PICK16S_12(...)
+#define QM_PICK16S_13(...)
 #if QM_TU == 0
 #undef QM_PICK16_0
 #define QM_PICK16_0(...) QM_TILE16_DEF(__VA_ARGS__)
@@ -167,6 +171,16 @@ static hipError_t launch_tiled_persistent(Kernel kernel, const GemmArgs &p, hipS
 #define QM_PICK16_11(...) QM_TILE16_DEF(__VA_ARGS__)
 #undef QM_PICK16S_11
 #define QM_PICK16S_11(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 12
+#undef QM_PICK16_12
+#define QM_PICK16_12(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_12
+#define QM_PICK16S_12(...) QM_TILE16S_DEF(__VA_ARGS__)
+#elif QM_TU == 13
+#undef QM_PICK16_13
+#define QM_PICK16_13(...) QM_TILE16_DEF(__VA_ARGS__)
+#undef QM_PICK16S_13
+#define QM_PICK16S_13(...) QM_TILE16S_DEF(__VA_ARGS__)
 #else
 #error "QM_TU out of range"
 #endif
